@@ -35,6 +35,13 @@ class BlockManager : public pk::BlockManagerCore {
     commit_prefix(seq, hashes.data(), tokens.data(), tokens.shape(0), std::min<int64_t>(n, hashes.shape(0)));
   }
 
+  // out[i] = state slot of seq_ids[i] (-1: none)
+  void state_slots_py(I64 seq_ids, I32 out) const {
+    const int64_t n = seq_ids.shape(0);
+    if (out.shape(0) < n) throw std::invalid_argument("state_slots: output too small");
+    for (int64_t i = 0; i < n; ++i) out.mutable_data()[i] = state_slot(seq_ids.data()[i]);
+  }
+
   int64_t pack_step(I64 seq_ids, I32 num_computed, I32 num_new, I32 tokens, I32 input_ids, I32 positions,
                     I32 slot_mapping, I32 block_tables, int max_blocks, I32 context_lens, I32 cu_q) {
     const int64_t n = seq_ids.shape(0);
@@ -60,8 +67,13 @@ PYBIND11_MODULE(_pk_runtime, m) {
   bind_step_channel(m);
   bind_vote_board(m);
   py::class_<BlockManager>(m, "BlockManager")
-      .def(py::init<int64_t, int, int64_t, bool, uint64_t>(), py::arg("num_blocks"), py::arg("block_size"),
-           py::arg("watermark_blocks") = 0, py::arg("prefix_caching") = false, py::arg("hash_key") = 0)
+      .def(py::init<int64_t, int, int64_t, bool, uint64_t, int64_t>(), py::arg("num_blocks"), py::arg("block_size"),
+           py::arg("watermark_blocks") = 0, py::arg("prefix_caching") = false, py::arg("hash_key") = 0,
+           py::arg("num_state_slots") = 0)
+      .def_property_readonly("num_state_slots", &BlockManager::num_state_slots)
+      .def_property_readonly("num_free_state_slots", &BlockManager::num_free_state_slots)
+      .def("state_slot", &BlockManager::state_slot)
+      .def("state_slots", &BlockManager::state_slots_py)
       .def_property_readonly("prefix_caching", &BlockManager::prefix_caching)
       .def_property_readonly("num_cached", &BlockManager::num_cached)
       .def_property_readonly("prefix_queries", &BlockManager::prefix_queries)

@@ -13,6 +13,12 @@
 // hash hit alone never shares a block -- match_prefix also requires the cached block's stored
 // tokens to equal the request's and its registered parent hash to equal the request's previous
 // block hash, so a forged 64-bit collision cannot serve one prompt another prompt's KV.
+//
+// State slots (optional, num_state_slots > 0): models whose layers carry a fixed-size state per
+// sequence beside the paged cache (the previous token's mixer input of a token-shift layer, a
+// recurrent state) keep it in slot-indexed device arrays.  A sequence takes a slot with its first
+// blocks and gives it back in free_seq; a sequence that cannot get one is not admitted.  A slot
+// is handed out as it was left: position 0 of a sequence never reads it.
 #pragma once
 #include <algorithm>
 #include <cstdint>
@@ -30,9 +36,14 @@ class BlockManagerCore {
  public:
   // hash_key 0: a random per-process key (tests pass a fixed one for reproducible hashes)
   BlockManagerCore(int64_t num_blocks, int block_size, int64_t watermark_blocks, bool prefix_caching = false,
-                   uint64_t hash_key = 0)
-      : num_blocks_(num_blocks), block_size_(block_size), watermark_(watermark_blocks), prefix_caching_(prefix_caching) {
+                   uint64_t hash_key = 0, int64_t num_state_slots = 0)
+      : num_blocks_(num_blocks), block_size_(block_size), watermark_(watermark_blocks), prefix_caching_(prefix_caching),
+        num_slots_(num_state_slots) {
     if (num_blocks <= 0 || block_size <= 0) throw std::invalid_argument("num_blocks and block_size must be > 0");
+    if (num_state_slots < 0) throw std::invalid_argument("num_state_slots must be >= 0");
+    if (num_state_slots > 0 && prefix_caching)
+      throw std::invalid_argument("a cached prefix has no per-sequence state: prefix caching needs num_state_slots == 0");
+    for (int64_t s = num_state_slots - 1; s >= 0; --s) free_slots_.push_back(static_cast<int32_t>(s));
     if (hash_key == 0) {
       std::random_device rd;
       hash_key = (static_cast<uint64_t>(rd()) << 32) ^ rd();
@@ -67,19 +78,37 @@ class BlockManagerCore {
     return std::max<int64_t>(0, blocks_for(total_tokens) - have);
   }
 
+  int64_t num_state_slots() const { return num_slots_; }
+  int64_t num_free_state_slots() const { return static_cast<int64_t>(free_slots_.size()); }
+  // the sequence's state slot, -1 if it has none
+  int32_t state_slot(int64_t seq) const {
+    auto it = slots_.find(seq);
+    return it == slots_.end() ? -1 : it->second;
+  }
+  bool slot_available(int64_t seq) const { return num_slots_ == 0 || slots_.count(seq) || !free_slots_.empty(); }
+
   bool can_allocate(int64_t seq, int64_t total_tokens, bool admission) const {
-    return needed(seq, total_tokens) + (admission ? watermark_ : 0) <= num_free();
+    return slot_available(seq) && needed(seq, total_tokens) + (admission ? watermark_ : 0) <= num_free();
   }
 
   bool allocate(int64_t seq, int64_t total_tokens) {
     const int64_t need = needed(seq, total_tokens);
-    if (need > num_free()) return false;
+    if (need > num_free() || !slot_available(seq)) return false;
+    if (num_slots_ > 0 && !slots_.count(seq)) {
+      slots_[seq] = free_slots_.back();
+      free_slots_.pop_back();
+    }
     auto& t = tables_[seq];
     for (int64_t i = 0; i < need; ++i) t.push_back(take_block());
     return true;
   }
 
   void free_seq(int64_t seq) {
+    auto sl = slots_.find(seq);
+    if (sl != slots_.end()) {
+      free_slots_.push_back(sl->second);
+      slots_.erase(sl);
+    }
     auto it = tables_.find(seq);
     if (it == tables_.end()) return;
     for (auto r = it->second.rbegin(); r != it->second.rend(); ++r) release(*r);
@@ -255,6 +284,9 @@ class BlockManagerCore {
   std::vector<char> in_lru_;
   std::unordered_map<uint64_t, int32_t> cached_;
   std::unordered_map<int64_t, std::vector<int32_t>> tables_;
+  int64_t num_slots_ = 0;
+  std::vector<int32_t> free_slots_;                 // stack: the slot freed last is taken first
+  std::unordered_map<int64_t, int32_t> slots_;      // sequence -> state slot
 };
 
 }  // namespace pk

@@ -77,7 +77,10 @@ class LLMEngine:
         self.st = st or get_state()
         mcfg: ModelConfig = get_config(cfg.model_path or cfg.model)
         if cfg.num_layers > 0 and cfg.num_layers != mcfg.num_layers:
-            mcfg = dataclasses.replace(mcfg, num_layers=cfg.num_layers)
+            if isinstance(mcfg, ModelConfig):
+                mcfg = dataclasses.replace(mcfg, num_layers=cfg.num_layers)
+            else:  # per-layer specs: keep the first num_layers of them
+                mcfg = dataclasses.replace(mcfg, layers=tuple(mcfg.layers[:cfg.num_layers]))
         if cfg.max_model_len > mcfg.max_position:
             cfg = dataclasses.replace(cfg, max_model_len=mcfg.max_position)
             self.cfg = cfg
@@ -131,7 +134,12 @@ class LLMEngine:
         self._serving_preflight(mcfg)
         nblocks = self.runner.allocate_kv_cache()
         rt = load_extension("_pk_runtime")
-        self.bm = rt.BlockManager(nblocks, cfg.block_size, int(nblocks * cfg.watermark), cfg.prefix_caching)
+        # per-sequence state beside the paged cache (token shift, recurrences): one slot per live
+        # sequence, handed out by the block manager; a cached prefix carries no such state, so
+        # these models run without prefix caching
+        stateful = bool(getattr(model, "needs_state", False))
+        self.bm = rt.BlockManager(nblocks, cfg.block_size, int(nblocks * cfg.watermark),
+                                  cfg.prefix_caching and not stateful, 0, cfg.max_num_seqs if stateful else 0)
         self.runner.bm = self.bm
         self.scheduler = Scheduler(self.bm, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.max_model_len,
                                    policy=cfg.sched_policy, max_decode_stall=cfg.max_decode_stall)
@@ -328,6 +336,54 @@ class LLMEngine:
         return [RequestOutput(s.request_id, [tok], reason is not None, reason.value if reason else None,
                               len(s.prompt_ids), len(s.output_ids), seq_metrics(s) if reason else None)
                 for s, tok, reason in done]
+
+    @torch.inference_mode()
+    def replay_step(self, entries, end=()) -> Optional[torch.Tensor]:
+        """One step of a recorded schedule, without sampling.  ``entries``: (request id, the
+        request's next tokens, places among them whose logits are wanted) -- a request is admitted
+        at its first entry and may sit out steps; all entries run as one batch through the
+        scheduler's forced step, the block manager and the model runner.  ``end``: requests
+        finished after this step (cache blocks and state slot freed).  Returns the fp32 logits
+        [wanted, vocab] in entry / place order, or None."""
+        sch = self.scheduler
+        plan = []
+        for rid, toks, _ in entries:
+            if not toks:
+                raise ValueError(f"request {rid}: empty entry")
+            if max(toks) >= self.mcfg.vocab_size or min(toks) < 0:
+                raise ValueError("token id out of range")
+            seq = sch.by_request.get(rid)
+            if seq is None:
+                seq = Sequence(rid, list(toks), SamplingParams(max_tokens=1), -1)
+                sch.by_request[rid] = seq
+            else:
+                seq.prompt_ids.extend(toks)
+            plan.append((seq, len(toks)))
+        logits = None
+        if plan:
+            batch = sch.schedule_forced(plan)
+            start, t = {}, 0
+            for s in batch.decodes:  # packed order: decodes, then the prefill portions
+                start[s.seq_id], t = t, t + 1
+            for s, n in batch.prefills:
+                start[s.seq_id], t = t, t + n
+            rows = []
+            for (seq, n), (_, _, want) in zip(plan, entries):
+                if any(w < 0 or w >= n for w in want):
+                    raise ValueError(f"request {seq.request_id}: wanted place outside the entry")
+                rows += [start[seq.seq_id] + w for w in want]
+            logits = self.runner.forward_logits(batch, rows)
+            for s, n in batch.prefills:
+                s.num_computed += n
+            for s in batch.decodes:
+                s.num_computed += 1
+            self.step_count += 1
+        for rid in end:
+            seq = sch.by_request.get(rid)
+            if seq is not None:
+                sch.finish(seq, FinishReason.STOP)
+        sch.remove_finished()
+        return logits
 
     def generate(self, prompts: List[List[int]], params: SamplingParams) -> List[List[int]]:
         seqs = [self.add_request(p, dataclasses.replace(params)) for p in prompts]

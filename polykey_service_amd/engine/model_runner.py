@@ -70,7 +70,10 @@ class _Layout:
         for name, n in (("header", 16), ("input_ids", max_tokens), ("positions", max_tokens), ("slots", max_tokens),
                         ("context_lens", max_seqs), ("cu_q", max_seqs + 1), ("cu_rel", max_seqs + 1), ("sample_idx", max_seqs),
                         ("temperature", max_seqs), ("top_k", max_seqs), ("top_p", max_seqs), ("min_p", max_seqs),
-                        ("seeds", max_seqs), ("offsets", max_seqs), ("block_tables", max_seqs * max_blocks)):
+                        ("seeds", max_seqs), ("offsets", max_seqs), ("block_tables", max_seqs * max_blocks),
+                        # whole-batch sections of own-cache models, behind the block tables so the
+                        # other families' per-step copy ends where it always did
+                        ("token_seq", max_tokens), ("state_slots", max_seqs), ("logit_rows", max_tokens)):
             self.sections[name] = (off, n)
             off += (n + 15) // 16 * 16  # 64-byte aligned sections
         self.size = off
@@ -125,17 +128,28 @@ class ModelRunner:
         self.graph_out: Dict[int, torch.Tensor] = {}
         self.short_graphs: Dict[int, torch.cuda.CUDAGraph] = {}
         self.short_graph_out: Dict[int, torch.Tensor] = {}
-        self.short_ctx = attn_ops._PART if cfg.max_model_len > attn_ops._PART else 0
+        # a model that lays out its own cache and per-sequence state (alloc_cache / needs_state):
+        # every sequence of the step is one varlen portion to its mixers, so the step metadata
+        # carries the whole-batch fields and the state slots
+        self.own_cache = hasattr(model, "alloc_cache")
+        self.stateful = bool(getattr(model, "needs_state", False))
+        self.short_ctx = attn_ops._PART if cfg.max_model_len > attn_ops._PART and not self.own_cache else 0
         self.graph_pool = None
-        a0 = model.layers[0].attn
-        self.part_o, self.part_ml = attn_ops.decode_workspace(cfg.max_num_seqs, a0.nq, self.max_blocks, self.bs, device,
-                                                              kv_heads=a0.nkv)
+        if self.own_cache:
+            self.part_o = self.part_ml = None
+            if hasattr(model, "reserve_steps"):
+                model.reserve_steps(self.max_step_tokens)
+        else:
+            a0 = model.layers[0].attn
+            self.part_o, self.part_ml = attn_ops.decode_workspace(cfg.max_num_seqs, a0.nq, self.max_blocks, self.bs,
+                                                                  device, kv_heads=a0.nkv)
         self.stats = {"steps": 0, "graph_steps": 0, "short_graph_steps": 0, "tokens": 0}
         self.keep_logits = False  # tests: keep the last eager step's logits
         self.last_logits = None
         # diagnostics (tools/tp_rehearsal.py): every step's logits, graphed steps included (a copy
         # captured into each graph); read last_logits right after the step, before the next one
         self.debug_logits = os.environ.get("POLYKEY_DEBUG_LOGITS") == "1"
+        self._graph_logits_kept = False  # capture_graphs(keep_logits=True): replays expose their logits
         self._graph_logits: Dict[Tuple[int, int], torch.Tensor] = {}
         self.channel = None
         self._prev_toks = None  # worker: last step's sampled ids (device), for continuations
@@ -167,11 +181,13 @@ class ModelRunner:
 
     # ---------------------------------------------------------------- KV cache
     def kv_bytes_per_block(self) -> int:
+        if self.own_cache:
+            return self.model.cache_bytes_per_block(self.bs)
         a = self.model.layers[0].attn
         return 2 * len(self.model.layers) * a.nkv * self.bs * a.hd * 2
 
     def allocate_kv_cache(self, num_blocks: int = 0) -> int:
-        a = self.model.layers[0].attn
+        a = None if self.own_cache else self.model.layers[0].attn
         if num_blocks <= 0:
             num_blocks = self.cfg.num_kv_blocks
         if num_blocks <= 0:
@@ -186,6 +202,9 @@ class ModelRunner:
             else:
                 num_blocks = max(16, min(self.cfg.max_num_seqs * self.max_blocks, 4096))
         self.num_blocks = num_blocks
+        if self.own_cache:
+            self.kv_caches = self.model.alloc_cache(num_blocks, self.bs, self.cfg.max_num_seqs if self.stateful else 0)
+            return num_blocks
         self.kv_caches = []
         for _ in self.model.layers:
             k = torch.zeros((num_blocks, a.nkv, self.bs, a.hd), dtype=self.model.dtype, device=self.device)
@@ -196,6 +215,10 @@ class ModelRunner:
     def activation_reserve_bytes(self) -> int:
         m = self.mcfg
         T = self.max_step_tokens
+        if self.own_cache:
+            state = self.model.state_bytes_per_slot() * self.cfg.max_num_seqs if self.stateful else 0
+            return int(T * self.model.activation_bytes_per_token() * 1.5 + state
+                       + self.cfg.max_num_seqs * m.vocab_size * 8 + (1 << 30))
         tp = self.model.st.tp_size
         per_tok = 2 * (m.hidden_size * 4 + (m.q_size + 2 * m.kv_size) // tp + 3 * m.intermediate_size // tp)
         logits = self.cfg.max_num_seqs * m.vocab_size * 4 * 2
@@ -221,6 +244,7 @@ class ModelRunner:
         h = self.h
         T = self.bm.pack_step(sids, ncomp, nnew, tok_arr, h["input_ids"], h["positions"], h["slots"],
                               h["block_tables"], self.max_blocks, h["context_lens"], h["cu_q"])
+        self._pack_whole_batch(sids, nnew, n)
         # sampling rows: hidden-state row index of each sampling sequence
         pos_of = {s.seq_id: int(h["cu_q"][i + 1]) - 1 for i, s in enumerate(seqs)}
         for r, s in enumerate(sampling):
@@ -234,6 +258,18 @@ class ModelRunner:
             h["offsets"][r] = len(s.output_ids)
         return T, n
 
+    def _pack_whole_batch(self, sids: np.ndarray, nnew: np.ndarray, n: int) -> None:
+        """Own-cache models: each token's sequence index and each sequence's state slot."""
+        if not self.own_cache:
+            return
+        h = self.h
+        T = int(h["cu_q"][n])
+        h["token_seq"][:T] = np.repeat(np.arange(n, dtype=np.int32), nnew[:n])
+        if self.stateful:
+            self.bm.state_slots(sids, h["state_slots"])
+        else:
+            h["state_slots"][:n] = -1
+
     def _metadata(self, nd: int, n: int, T: int, max_q: int, short: bool = False) -> attn_ops.AttnMetadata:
         """``short``: every decode context is at most ``self.short_ctx`` tokens."""
         d = self.d
@@ -245,6 +281,9 @@ class ModelRunner:
             decode_context_lens=d["context_lens"][:nd] if nd else None,
             decode_part_o=self.part_o, decode_part_ml=self.part_ml,
             decode_max_ctx=self.short_ctx if short else 0)
+        if self.own_cache:
+            md.num_seqs, md.cu_q, md.context_lens = n, d["cu_q"][:n + 1], d["context_lens"][:n]
+            md.block_tables, md.token_seq, md.state_slots = d["block_tables"][:n], d["token_seq"][:T], d["state_slots"][:n]
         if npf:
             md.prefill_block_tables = d["block_tables"][nd:n]
             md.prefill_context_lens = d["context_lens"][nd:n]
@@ -299,6 +338,48 @@ class ModelRunner:
         self._publish(max(n, g))
         toks = self._run(T, n, nd, ns, max_q, g, short)
         return self._handle(toks, ns)
+
+    @torch.inference_mode()
+    def forward_logits(self, batch: ScheduledBatch, rows: List[int]) -> Optional[torch.Tensor]:
+        """One step without sampling: pack, stage and run ``batch`` like :meth:`launch`, and return
+        the fp32 logits at token rows ``rows`` of the packed step (decodes first, then the prefill
+        portions in order) on the host; None when no row is asked.  A pure-decode step whose rows
+        are exactly its sequences replays the captured decode graph like generation does."""
+        if self.model.st.tp_size > 1:
+            raise NotImplementedError("forward_logits: single-rank engines only")
+        self._next_staging()
+        T, n = self._pack(batch, [])
+        nd = len(batch.decodes)
+        h, d = self.h, self.d
+        if any(r < 0 or r >= T for r in rows):
+            raise ValueError("logit row outside the step")
+        max_q = g = 0
+        if batch.prefills:
+            rel = h["cu_q"][nd:n + 1] - h["cu_q"][nd]
+            h["cu_rel"][:n - nd + 1] = rel
+            max_q = int(np.max(np.diff(rel)))
+        elif self.graphs and self.allow_graphs and rows == list(range(nd)) and self._graph_logits_kept:
+            g = self._graph_bucket(nd) or 0
+            if g:
+                self._pad_decode(nd, g)
+        short = self._short(g, nd)
+        nr = len(rows)
+        h["logit_rows"][:nr] = rows
+        h["header"][:9] = (self.MODE_RUN, T, n, nd, 0, max_q, g, short, 0)
+        self._publish(max(n, g))
+        self.stats["steps"] += 1
+        if g:
+            self._run(T, n, nd, nd, 0, g, short)
+            self.last_logits = self._graph_logits[(g, int(bool(short)))]
+            return self.last_logits[:nd].float().cpu()
+        md = self._metadata(nd, n, T, max_q, bool(short))
+        hidden = self.model(d["input_ids"][:T], d["positions"][:T], md, self.kv_caches)
+        if nr == 0:
+            if self.device.type == "cuda":
+                torch.cuda.current_stream(self.device).synchronize()
+            return None
+        logits = self.model.compute_logits(hidden.index_select(0, d["logit_rows"][:nr].long()))
+        return logits.float().cpu()
 
     def _short(self, g: int, nd: int) -> int:
         """1 when every decode context fits one attention partition: the step replays bucket
@@ -367,6 +448,7 @@ class ModelRunner:
         ones = np.ones(n, dtype=np.int32)
         T = self.bm.pack_step(sids, ncomp, ones, np.zeros(n, dtype=np.int32), h["input_ids"], h["positions"],
                               h["slots"], h["block_tables"], self.max_blocks, h["context_lens"], h["cu_q"])
+        self._pack_whole_batch(sids, ones, n)
         h["sample_idx"][:n] = np.arange(n, dtype=np.int32)
         for r, s in enumerate(seqs):
             p = s.params
@@ -386,6 +468,8 @@ class ModelRunner:
     def _staged_words(self, n_bt_rows: Optional[int]) -> int:
         """int32 words of the staging buffer a step uses: everything up to the used block-table
         rows (the last section), rounded to 16 bytes."""
+        if self.own_cache:
+            return self.layout.size
         off, _ = self.layout.sections["block_tables"]
         rows = self.cfg.max_num_seqs if n_bt_rows is None else n_bt_rows
         n = min(self.layout.size, off + rows * self.max_blocks)
@@ -564,6 +648,10 @@ class ModelRunner:
             h["top_k"][nd:g] = 0
             h["top_p"][nd:g] = 1.0
             h["min_p"][nd:g] = 0.0
+            if self.own_cache:  # padded rows: one-token sequences at position 0 without cache or state
+                h["cu_q"][nd + 1:g + 1] = np.arange(nd + 1, g + 1, dtype=np.int32)
+                h["token_seq"][nd:g] = np.arange(nd, g, dtype=np.int32)
+                h["state_slots"][nd:g] = -1
 
     def default_graph_sizes(self) -> List[int]:
         if self.cfg.graph_batch_sizes:
@@ -573,9 +661,12 @@ class ModelRunner:
         return [s for s in sizes if s <= self.cfg.max_num_seqs]
 
     @torch.inference_mode()
-    def capture_graphs(self, sizes: Optional[List[int]] = None) -> None:
+    def capture_graphs(self, sizes: Optional[List[int]] = None, keep_logits: bool = False) -> None:
+        """``keep_logits``: each graph's logits tensor stays referenced (it lives in the graph's
+        memory pool), so a replay's logits can be read (:meth:`forward_logits`)."""
         if self.device.type != "cuda" or not self.cfg.hip_graphs:
             return
+        self._graph_logits_kept = keep_logits or self.debug_logits
         sizes = sizes or self.default_graph_sizes()
         st = self.model.st
         if st.dp_attention:  # every replay sends bucket x top-k rows per peer: within the IPC capacity
@@ -588,6 +679,11 @@ class ModelRunner:
         self.h["context_lens"][: self.cfg.max_num_seqs] = 1
         self.h["top_p"][:] = 1.0
         self.h["sample_idx"][: self.cfg.max_num_seqs] = np.arange(self.cfg.max_num_seqs, dtype=np.int32)
+        if self.own_cache:
+            self.h["cu_q"][: self.cfg.max_num_seqs + 1] = np.arange(self.cfg.max_num_seqs + 1, dtype=np.int32)
+            self.h["token_seq"][: self.cfg.max_num_seqs] = np.arange(self.cfg.max_num_seqs, dtype=np.int32)
+            self.h["state_slots"][:] = -1
+            self.h["context_lens"][: self.cfg.max_num_seqs] = 0
         self.dev_buf.copy_(self.host_buf)
         torch.cuda.synchronize(self.device)
         stream = torch.cuda.Stream(self.device)
@@ -603,6 +699,8 @@ class ModelRunner:
                 logits = self.model.compute_logits(hidden)
                 if self.debug_logits:
                     self._graph_logits[(g, int(short))] = logits.clone()
+                elif keep_logits:
+                    self._graph_logits[(g, int(short))] = logits
                 return sampler_ops.sample(logits, d["temperature"][:g], d["top_k"][:g], d["top_p"][:g],
                                           d["min_p"][:g], d["seeds"][:g], d["offsets"][:g])
 

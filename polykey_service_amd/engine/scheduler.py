@@ -217,6 +217,40 @@ class Scheduler:
         self._decode_stall = self._decode_stall + 1 if skipped else 0
         return ScheduledBatch(st.decodes, st.prefills, st.preempted)
 
+    def schedule_forced(self, plan: List[Tuple[Sequence, int]]) -> ScheduledBatch:
+        """A step whose contents the caller dictates (replaying a recorded schedule): each
+        (sequence, n) runs its next n tokens.  Admission and cache growth go through the same
+        block manager calls as :meth:`schedule`; nothing is preempted -- a step that does not fit
+        the pool, the state slots or the sequence cap is an error of the schedule."""
+        if sum(n for _, n in plan) > self.max_num_batched_tokens:
+            raise ValueError(f"step of {sum(n for _, n in plan)} tokens exceeds the budget {self.max_num_batched_tokens}")
+        decodes: List[Sequence] = []
+        prefills: List[Tuple[Sequence, int]] = []
+        for seq, n in plan:
+            if n < 1 or n > seq.num_pending:
+                raise ValueError(f"request {seq.request_id}: {n} tokens asked, {seq.num_pending} pending")
+            if seq.num_computed + n > self.max_model_len:
+                raise ValueError(f"request {seq.request_id} exceeds max_model_len {self.max_model_len}")
+            new = seq.status == SeqStatus.WAITING
+            if new and len(self.running) >= self.max_num_seqs:
+                raise RuntimeError(f"more than {self.max_num_seqs} live sequences")
+            if not self.bm.allocate(seq.seq_id, seq.num_computed + n):
+                raise RuntimeError(f"request {seq.request_id}: the cache pool or the state slots are exhausted")
+            if new:
+                try:
+                    self.waiting.remove(seq)
+                except ValueError:
+                    pass
+                seq.status = SeqStatus.RUNNING
+                seq.first_scheduled = time.monotonic()
+                bisect.insort(self.running, seq, key=lambda s: s.seq_id)
+                self.by_request[seq.request_id] = seq
+            if n == 1 and seq.num_computed > 0:
+                decodes.append(seq)
+            else:
+                prefills.append((seq, n))
+        return ScheduledBatch(decodes, prefills, [])
+
     def _schedule_running(self, st: "_Step") -> None:
         i = 0
         while i < len(self.running) and st.budget > 0:

@@ -86,11 +86,113 @@ PRESETS: Dict[str, ModelConfig] = {
 }
 
 
-def get_config(name_or_path: str) -> ModelConfig:
+@dataclasses.dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose keys and values are expanded from one cached low-rank latent per token."""
+    heads: int
+    dim: int        # query / key size per head
+    vdim: int       # value size per head
+    kv_rank: int    # size of the cached latent
+    scale: float
+
+
+@dataclasses.dataclass(frozen=True)
+class SigmoidMoESpec:
+    """Experts chosen by the largest sigmoid(router) scores; the score scales the expert's input."""
+    experts: int
+    top: int
+    ff: int
+
+
+@dataclasses.dataclass(frozen=True)
+class LayerSpec:
+    type: str
+    mixer: LatentAttentionSpec
+    mlp: Optional[SigmoidMoESpec]
+
+
+@dataclasses.dataclass(frozen=True)
+class SapapelConfig:
+    """Sapapel: post-norm layers (one scalar gain per norm, alpha-scaled skip path) with a token
+    shift in front of each mixer, a learned average over all earlier layers' outputs behind each
+    layer, latent attention without positions and a sigmoid-routed MoE.  Read from a checkpoint
+    folder's config.json ("architecture": "Sapapel"); every size comes from there."""
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple
+    alpha: float
+    rms_eps: float
+    max_position: int = 1 << 20     # no positional encoding: bounded by the cache only
+    bos_token_id: int = 0
+    eos_token_id: int = -1          # the checkpoint names no end token
+    init_std: float = 0.05
+    family: str = "sapapel"
+    is_moe: bool = False            # not the Mixtral expert-parallel family (engine lockstep paths)
+    experts_per_token: int = 0
+    needs_state: bool = True        # per-sequence token-shift state beside the paged cache
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def num_params(self) -> int:
+        W, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size
+        for l in self.layers:
+            m = l.mixer
+            n += W * (m.heads * m.dim + m.kv_rank + 2 * m.heads * m.vdim) + m.kv_rank * m.heads * (m.dim + m.vdim)
+            if l.mlp is not None:
+                n += l.mlp.experts * (3 * l.mlp.ff * W + W)
+        return n
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        return sum(l.mixer.kv_rank for l in self.layers) * dtype_bytes
+
+    @classmethod
+    def from_json(cls, c: dict, name: str = "sapapel") -> "SapapelConfig":
+        layers = []
+        for l in c["layers"]:
+            if l["type"] != "latent_attention":
+                raise ValueError(f"Sapapel: unknown mixer type {l['type']!r}")
+            m = l["mixer"]
+            mixer = LatentAttentionSpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), int(m["kv_rank"]),
+                                        float(m["scale"]))
+            f = l.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind") != "moe":
+                    raise ValueError(f"Sapapel: unknown feed-forward kind {f.get('kind')!r}")
+                mlp = SigmoidMoESpec(int(f["router"]["experts"]), int(f["router"]["top"]), int(f["expert"]["ff"]))
+            layers.append(LayerSpec(l["type"], mixer, mlp))
+        return cls(name=name, vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), layers=tuple(layers),
+                   alpha=float(c["postln_alpha"]), rms_eps=float(c["norm"]["eps"]))
+
+    @classmethod
+    def uniform(cls, name: str, vocab: int, width: int, n_layers: int, heads: int, dim: int, vdim: int, kv_rank: int,
+                ff: int, experts: int, top: int, alpha: float = 2.0, eps: float = 1e-6) -> "SapapelConfig":
+        l = LayerSpec("latent_attention", LatentAttentionSpec(heads, dim, vdim, kv_rank, dim ** -0.5),
+                      SigmoidMoESpec(experts, top, ff))
+        return cls(name=name, vocab_size=vocab, hidden_size=width, layers=(l,) * n_layers, alpha=alpha, rms_eps=eps)
+
+
+# config.json "architecture" -> reader (checkpoints that are not HF Llama / Mixtral folders)
+ARCHITECTURES = {"Sapapel": SapapelConfig.from_json}
+
+PRESETS["tiny-sapapel"] = SapapelConfig.uniform("tiny-sapapel", 512, 128, 3, 4, 16, 32, 48, 64, 6, 2)
+# layer shapes of a ~1B-active latent-attention MoE (random weights; speed measurements)
+PRESETS["sapapel-2k"] = SapapelConfig.uniform("sapapel-2k", 32000, 2048, 8, 16, 128, 128, 512, 1408, 16, 2)
+
+
+def get_config(name_or_path: str):
     if name_or_path in PRESETS:
         return PRESETS[name_or_path]
     path = os.path.join(name_or_path, "config.json") if os.path.isdir(name_or_path) else name_or_path
     if os.path.isfile(path):
+        with open(path) as f:
+            arch = json.load(f).get("architecture")
+        if arch in ARCHITECTURES:
+            with open(path) as f:
+                return ARCHITECTURES[arch](json.load(f), os.path.basename(os.path.dirname(os.path.abspath(path))) or arch)
         return from_hf_config(path)
     raise KeyError(f"unknown model {name_or_path!r}; presets: {sorted(PRESETS)}")
 

@@ -33,6 +33,14 @@ class AttnMetadata:
     decode_part_o: Optional[torch.Tensor] = None         # split-K workspace
     decode_part_ml: Optional[torch.Tensor] = None
     decode_max_ctx: int = 0  # bound on every decode context of the step (0: block-table capacity)
+    # whole-batch view (decodes first, then prefills) for mixers that treat every sequence as a
+    # varlen portion, and per-sequence state slots (models with state beside the paged cache)
+    num_seqs: int = 0
+    cu_q: Optional[torch.Tensor] = None            # [n+1] int32 token offsets of the step's sequences
+    context_lens: Optional[torch.Tensor] = None    # [n] int32 cached tokens after this step
+    block_tables: Optional[torch.Tensor] = None    # [n, MB] int32
+    token_seq: Optional[torch.Tensor] = None       # [T] int32 batch index of each token's sequence
+    state_slots: Optional[torch.Tensor] = None     # [n] int32 (-1: none)
 
     @property
     def num_tokens(self) -> int:

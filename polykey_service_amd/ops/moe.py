@@ -64,6 +64,11 @@ def align(ids: torch.Tensor, E: int, e_lo: int, e_hi: int):
     offsets = torch.empty(El + 1, dtype=torch.int32, device=dev)
     sorted_ = torch.empty(n, dtype=torch.int32, device=dev)
     inv = torch.empty(n, dtype=torch.int32, device=dev)
+    if El > 64:  # beyond the single-wave stable sort: the LDS-counter align (all experts local)
+        assert e_lo == 0 and e_hi == E
+        native.call("pkm_expert_align_wide", ids.data_ptr(), offsets.data_ptr(), sorted_.data_ptr(), inv.data_ptr(), n,
+                    E, native.stream_ptr())
+        return offsets, sorted_, inv
     native.call("pk_moe_align", ids.data_ptr(), offsets.data_ptr(), sorted_.data_ptr(), inv.data_ptr(), n, E, e_lo,
                 e_hi, native.stream_ptr())
     return offsets, sorted_, inv
@@ -209,4 +214,62 @@ def fused_moe_reference(x, router_w, w13, w2, k, e_lo=0, e_hi=None):
         y = bf(h @ w2[e - e_lo].float().t())
         sel = (ids == e).float() * w
         out += sel.sum(-1, keepdim=True) * y
+    return out
+
+
+# ------------------------------------------------------------------ sigmoid-routed, input-scaled MoE
+def route_sigmoid_topk(x: torch.Tensor, router_w: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp32 router: s = sigmoid(router_w x); the k largest s per token and their experts (ties: the
+    lower expert id), scores as they are.  x [T, W] fp32, router_w [E, W] fp32."""
+    T, W = x.shape
+    E = router_w.shape[0]
+    if not x.is_cuda:
+        s = torch.sigmoid(x.float() @ router_w.float().t())
+        w, ids = torch.sort(s, dim=-1, descending=True, stable=True)
+        return ids[:, :k].to(torch.int32).contiguous(), w[:, :k].contiguous()
+    assert x.dtype == torch.float32 and router_w.dtype == torch.float32 and x.is_contiguous()
+    ids = torch.empty((T, k), dtype=torch.int32, device=x.device)
+    w = torch.empty((T, k), dtype=torch.float32, device=x.device)
+    native.call("pkm_route_sigmoid_topk", ids.data_ptr(), w.data_ptr(), x.data_ptr(), router_w.data_ptr(), T, W, E, k,
+                native.stream_ptr())
+    return ids, w
+
+
+def input_scaled_moe(x_act: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+                     down: torch.Tensor) -> torch.Tensor:
+    """sum over a token's experts of down_e(silu(gate_e(s x)) * up_e(s x)), s the expert's score,
+    as fp32 [T, W].  x_act [T, W] in the weights' dtype; gate / up [E, F, W]; down [E, W, F].
+    Tokens are grouped by expert on the device (align), the score is applied to the gate / up
+    products, and the combine is a plain sum."""
+    T, W = x_act.shape
+    E, F_, _ = gate.shape
+    k = ids.shape[1]
+    offsets, sorted_, inv = align(ids, E, 0, E)
+    if not x_act.is_cuda:
+        m = int(offsets[-1])
+        tok = sorted_[:m].long() // k
+        s = wts.reshape(-1)[sorted_[:m].long()].float()
+        y = torch.zeros((m, W), dtype=torch.float32)
+        offs = offsets.tolist()
+        for e in range(E):
+            lo, hi = offs[e], offs[e + 1]
+            if hi > lo:
+                xe = x_act[tok[lo:hi]].float()
+                g = (xe @ gate[e].float().t()) * s[lo:hi, None]
+                u = (xe @ up[e].float().t()) * s[lo:hi, None]
+                h = (g * torch.sigmoid(g) * u).to(x_act.dtype).float()
+                y[lo:hi] = h @ down[e].float().t()
+        return y[inv.long().view(T, k)].sum(1)
+    assert x_act.is_contiguous() and gate.is_contiguous() and up.is_contiguous() and down.is_contiguous()
+    assert gate.dtype == x_act.dtype and wts.dtype == torch.float32 and wts.is_contiguous()
+    dt = native.dt_code(x_act.dtype)
+    n = T * k
+    h = torch.empty((n, F_), dtype=x_act.dtype, device=x_act.device)
+    y = torch.empty((n, W), dtype=torch.float32, device=x_act.device)
+    out = torch.empty((T, W), dtype=torch.float32, device=x_act.device)
+    st = native.stream_ptr()
+    native.call("pkm_expert_gate_up", h.data_ptr(), x_act.data_ptr(), gate.data_ptr(), up.data_ptr(), offsets.data_ptr(),
+                sorted_.data_ptr(), wts.data_ptr(), n, k, E, F_, W, dt, st)
+    native.call("pkm_expert_down", y.data_ptr(), h.data_ptr(), down.data_ptr(), offsets.data_ptr(), n, E, W, F_, dt, st)
+    native.call("pkm_combine_rows", out.data_ptr(), y.data_ptr(), inv.data_ptr(), T, k, W, st)
     return out

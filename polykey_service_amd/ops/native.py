@@ -66,6 +66,48 @@ SIGNATURES = {
 }
 
 
+# libpk_mixers (csrc/mixers): kernels built for bf16 and fp32 element types (``dt``: 0 bf16, 1 fp32)
+MIXER_SIGNATURES = {
+    "pkm_abi_version": [],
+    "pkm_embed_rows": [P, P, P, I32, I32, I32, I32, P],
+    "pkm_token_shift": [P, P, P, P, P, P, P, P, I32, I32, I32, P],
+    "pkm_save_last_rows": [P, P, P, P, I32, I32, P],
+    "pkm_sum_gain_norm": [P, P, P, P, P, F32, P, F32, I32, I32, P, I64, I32, P, I32, I32, P],
+    "pkm_latent_norm_cache": [P, P, I64, P, P, I32, I32, F32, I32, P],
+    "pkm_latent_attention": [P, I64, I64, P, I64, I64, P, P, I32, P, P, I32, I32, I32, I32, I32, F32, I32, P],
+    "pkm_gate_merge": [P, P, I64, I64, P, I64, I32, I32, I32, I32, P],
+    "pkm_route_sigmoid_topk": [P, P, P, P, I32, I32, I32, I32, P],
+    "pkm_expert_gate_up": [P, P, P, P, P, P, P, I32, I32, I32, I32, I32, I32, P],
+    "pkm_expert_down": [P, P, P, P, I32, I32, I32, I32, I32, P],
+    "pkm_combine_rows": [P, P, P, I32, I32, I32, P],
+    "pkm_expert_align_wide": [P, P, P, P, I32, I32, P],
+}
+_mixers: Optional[ctypes.CDLL] = None
+
+
+def mixers() -> ctypes.CDLL:
+    global _mixers
+    if _mixers is None:
+        with _lock:
+            if _mixers is None:
+                l = load_cdll("libpk_mixers")
+                for name, argtypes in MIXER_SIGNATURES.items():
+                    fn = getattr(l, name)
+                    fn.argtypes = argtypes
+                    fn.restype = ctypes.c_int
+                _mixers = l
+    return _mixers
+
+
+def dt_code(dtype: torch.dtype) -> int:
+    """Element-type code of the libpk_mixers launchers."""
+    if dtype == torch.bfloat16:
+        return 0
+    if dtype == torch.float32:
+        return 1
+    raise TypeError(f"the mixer kernels are built for bfloat16 and float32, not {dtype}")
+
+
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
@@ -105,5 +147,5 @@ def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 def call(name: str, *args) -> None:
-    fn = getattr(lib(), name)
+    fn = getattr(mixers() if name in MIXER_SIGNATURES else lib(), name)
     check(fn(*args), name)
