@@ -104,23 +104,26 @@ def random_model(cfg: dict, seed: int = 0, std: float = 0.08) -> Dict[str, torch
     def r(*shape, s=std):
         return (torch.randn(*shape, generator=g) * s).bfloat16().float()
 
-    w = {"embed": r(cfg["vocab"], W, s=1.0), "final.norm": (1 + r(1, s=0.1))[0], "head": r(cfg["vocab"], W)}
+    def gain(*shape):  # near 1, and exact in bf16 like everything a checkpoint holds
+        return (1 + torch.randn(*shape, generator=g) * 0.1).bfloat16().float()
+
+    w = {"embed": r(cfg["vocab"], W, s=1.0), "final.norm": gain(1)[0], "head": r(cfg["vocab"], W)}
     for i, lc in enumerate(cfg["layers"]):
         p, m = f"l{i}.", lc["mixer"]
         H, D, V, R = m["heads"], m["dim"], m["vdim"], m["kv_rank"]
-        w[p + "norm1"] = (1 + r(1, s=0.1))[0]
+        w[p + "norm1"] = gain(1)[0]
         w[p + "shift"] = torch.rand(W, generator=g).bfloat16().float()
         w[p + "dwa"] = (torch.eye(i + 2)[i + 1] * 0.7 + r(i + 2, s=0.2)).bfloat16().float()
         w[p + "mix.q"] = r(H * D, W)
         w[p + "mix.dkv"] = r(R, W)
-        w[p + "mix.dkv.norm"] = (1 + r(R, s=0.1))
+        w[p + "mix.dkv.norm"] = gain(R)
         w[p + "mix.uk"] = r(H * D, R, s=std * 2)
         w[p + "mix.uv"] = r(H * V, R, s=std * 2)
         w[p + "mix.g"] = r(H * V, W)
         w[p + "mix.o"] = r(W, H * V)
         f = lc.get("mlp")
         if f is not None:
-            w[p + "norm2"] = (1 + r(1, s=0.1))[0]
+            w[p + "norm2"] = gain(1)[0]
             w[p + "mlp.router"] = r(f["router"]["experts"], W, s=0.5)
             for e in range(f["router"]["experts"]):
                 F = f["expert"]["ff"]
