@@ -99,6 +99,13 @@ def parse_args(argv=None):
                     help="N > 1: seconds the whole run may take, below the driver's 600 s command limit. The main "
                          "child gets at most this minus a print margin, the TP child only what is left, so the "
                          "JSON line is always printed in time")
+    ap.add_argument("--compare-families", default="",
+                    help="instead of the headline workload: engine-level prefill and decode throughput of the "
+                         "Sapapel family beside the Mixtral family at equal layer sizes, e.g. '2k,4k' "
+                         "(presets sapapel-<size> / mixtral-<size>; random weights, one GPU, no RPC)")
+    ap.add_argument("--compare-batch", type=int, default=32, help="--compare-families: sequences")
+    ap.add_argument("--compare-prompt", type=int, default=1024, help="--compare-families: prompt tokens per sequence")
+    ap.add_argument("--compare-decode", type=int, default=128, help="--compare-families: decoded tokens per sequence")
     ap.add_argument("--child", action="store_true", help=argparse.SUPPRESS)  # internal: the measuring torchrun job
     return ap.parse_args(argv)
 
@@ -463,9 +470,63 @@ async def _drive_external(args, engine, st, leaders_group, port, srv, llm, conc,
     return res["tokens"], elapsed, res["lats"]
 
 
+def compare_families(args) -> int:
+    """Prefill and decode throughput of one engine per (family, size), the same requests for both
+    families: B prompts of S random tokens prefilled under the engine's token budget, then K
+    decode steps of all B sequences (HIP-graph replays).  One JSON line per engine."""
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import torch
+
+    from polykey_service_amd.engine import EngineConfig, LLMEngine, SamplingParams
+    from polykey_service_amd.parallel.state import ParallelState
+
+    dev = torch.device("cuda:0")
+    B, S, K = args.compare_batch, args.compare_prompt, args.compare_decode
+    max_len = (S + K + 64 + 511) // 512 * 512
+    rng = __import__("random").Random(args.seed)
+    for item in [x for x in args.compare_families.split(",") if x]:
+        size, _, only = item.partition(":")  # "2k" both families, "2k:sapapel" one (profiling)
+        for fam in ((only,) if only else ("sapapel", "mixtral")):
+            name = f"{fam}-{size}"
+            eng = LLMEngine(EngineConfig(model=name, seed=args.seed, max_num_seqs=B,
+                                         max_num_batched_tokens=args.max_batched_tokens, max_model_len=max_len,
+                                         hip_graphs=not args.no_graphs, graph_batch_sizes=(B,), prefix_caching=False,
+                                         num_kv_blocks=B * (max_len // 32) + 16), ParallelState(device=dev))
+            V = eng.mcfg.vocab_size
+            prompts = [[rng.randrange(3, V) for _ in range(S)] for _ in range(B)]
+            eng.generate([p[:96] for p in prompts[:2]], SamplingParams(max_tokens=4, ignore_eos=True))  # warm-up
+            torch.cuda.synchronize(dev)
+            t0 = time.perf_counter()
+            eng.generate(prompts, SamplingParams(max_tokens=1, ignore_eos=True))
+            torch.cuda.synchronize(dev)
+            t_prefill = time.perf_counter() - t0
+            seqs = [eng.add_request(p, SamplingParams(max_tokens=K + 1, ignore_eos=True)) for p in prompts]
+            while any(not s.output_ids for s in seqs):
+                eng.step()
+            torch.cuda.synchronize(dev)
+            steps0 = eng.step_count
+            t0 = time.perf_counter()
+            while eng.has_unfinished():
+                eng.step()
+            torch.cuda.synchronize(dev)
+            t_decode = time.perf_counter() - t0
+            n_dec = sum(len(s.output_ids) - 1 for s in seqs)
+            print(json.dumps({"metric": "family_compare", "model": name, "params": eng.mcfg.num_params(),
+                              "batch": B, "prompt_len": S, "decode_len": K, "dtype": "bf16", "data": "synthetic",
+                              "prefill_tok_s": round(B * S / t_prefill, 1), "decode_tok_s": round(n_dec / t_decode, 1),
+                              "decode_ms_per_step": round(1e3 * t_decode / max(eng.step_count - steps0, 1), 3),
+                              "graph_steps": eng.runner.stats["graph_steps"]}), flush=True)
+            eng.shutdown()
+            del eng
+            torch.cuda.empty_cache()
+    return 0
+
+
 def main(argv=None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
     args = parse_args(argv)
+    if args.compare_families:
+        return compare_families(args)
     if args.gpus > 1 and not args.child:
         if int(os.environ.get("RANK", "0")) != 0:
             return 0  # under the driver's torchrun: rank 0 runs the measurement children

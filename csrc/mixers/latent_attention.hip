@@ -22,10 +22,16 @@ using namespace pkm;
 
 namespace {
 
+// column of key k (0..31) inside a 32-key tile of the latent-major copy: the key-slot order of the
+// matrix-core kernels' second product (see latent_attention_mfma_kernel)
+__host__ __device__ __forceinline__ int key_slot(int k) { return ((k & 15) >> 2) * 8 + (k & 3) + 4 * (k >> 4); }
+
+// cache_t (optional): the latent-major copy [blocks][block_size / 32][R][32 key slots]
 template <typename T>
 __global__ void __launch_bounds__(128)
-latent_norm_cache_kernel(T* __restrict__ cache, const T* __restrict__ dkv, int64_t dkv_stride,
-                         const float* __restrict__ w, const int* __restrict__ slot_mapping, int R, float eps) {
+latent_norm_cache_kernel(T* __restrict__ cache, T* __restrict__ cache_t, int block_size, const T* __restrict__ dkv,
+                         int64_t dkv_stride, const float* __restrict__ w, const int* __restrict__ slot_mapping, int R,
+                         float eps) {
   __shared__ float red[16];
   const int t = blockIdx.x;
   const int slot = slot_mapping[t];
@@ -39,7 +45,16 @@ latent_norm_cache_kernel(T* __restrict__ cache, const T* __restrict__ dkv, int64
   if (slot < 0) return;
   const float k = 1.f / sqrtf(ss / static_cast<float>(R) + eps);
   T* dst = cache + static_cast<int64_t>(slot) * R;
-  for (int i = threadIdx.x; i < R; i += blockDim.x) st<T>(dst + i, ld<T>(src + i) * k * w[i]);
+  T* dst_t = nullptr;
+  if (cache_t) {
+    const int kb = slot % block_size;
+    dst_t = cache_t + (static_cast<int64_t>(slot / block_size) * (block_size / 32) + kb / 32) * R * 32 + key_slot(kb & 31);
+  }
+  for (int i = threadIdx.x; i < R; i += blockDim.x) {
+    const float v = ld<T>(src + i) * k * w[i];
+    st<T>(dst + i, v);
+    if (dst_t) st<T>(dst_t + static_cast<int64_t>(i) * 32, v);
+  }
 }
 
 constexpr int kBQ = 16;       // (token, head) rows per workgroup
@@ -168,6 +183,313 @@ latent_attention_kernel(T* __restrict__ out, int64_t out_st, int64_t out_sh, con
   }
 }
 
+// ---- bf16 on the matrix cores -------------------------------------------------------------------
+// 64 (token, head) rows per workgroup, 16 per wave; 32-key tiles.  Both products run transposed on
+// mfma_f32_16x16x32_bf16 so that the softmax weights never leave their registers:
+//
+//   S^T [keys x rows] = C [keys x R] . Q~^T     A = key rows from LDS `cs`, B = the wave's Q~ (registers)
+//   O~^T [R x rows]  += C^T [R x keys] . P^T    A = latent rows from the transposed LDS copy `ct`,
+//                                               B = P^T straight from the S^T accumulators
+//
+// An accumulator lane (g, n) holds query row n and keys 4g..4g+3 of each 16-key half; the B operand
+// of the second product wants 8 key slots per lane, so slot (g, e) is key 4g+e of the first half
+// for e < 4 and key 16+4g+e-4 of the second, and `ct` stores its columns in that slot order.
+// The tile is staged twice (key-major and latent-major) because it is both the key and the value.
+template <int R>
+__global__ void __launch_bounds__(256)
+latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t out_sh, const bf16_t* __restrict__ q,
+                             int64_t q_st, int64_t q_sh, const bf16_t* __restrict__ cache,
+                             const bf16_t* __restrict__ cache_t, const int* __restrict__ block_tables, int max_blocks,
+                             const int* __restrict__ cu_q, const int* __restrict__ context_lens, int n_seqs, int H,
+                             int block_size, float scale) {
+  constexpr int BQ = 64, BK = 32, NKK = R / 32, NRT = R / 16, CS = R + 8, CT = BK + 8, R8 = R / 8;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16_t* cs = reinterpret_cast<bf16_t*>(smem_raw);  // [BK][CS]   key-major
+  bf16_t* ct = cs + BK * CS;                          // [R][CT]    latent-major, key slots permuted
+  int s = 0, tile = blockIdx.x;
+  for (; s < n_seqs; ++s) {
+    const int nt = ((cu_q[s + 1] - cu_q[s]) * H + BQ - 1) / BQ;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (s >= n_seqs) return;
+  const int q0 = cu_q[s], qlen = cu_q[s + 1] - q0, ctx = context_lens[s];
+  const int n_rows = qlen * H, row0 = tile * BQ;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, n = lane & 15;
+  const int* bt = block_tables + static_cast<int64_t>(s) * max_blocks;
+  const int my_row = row0 + 16 * wave + n;
+  const bool valid = my_row < n_rows;
+  const int tl = valid ? my_row / H : 0, h = valid ? my_row - tl * H : 0;
+  const int my_pos = valid ? ctx - qlen + tl : -1;
+  const int max_pos = ctx - qlen + (min(row0 + BQ, n_rows) - 1) / H;
+
+  pk::bf16x8_t qf[NKK];
+  {
+    const bf16_t* qr = q + static_cast<int64_t>(q0 + tl) * q_st + static_cast<int64_t>(h) * q_sh + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      pk::u32x4 v = {0u, 0u, 0u, 0u};
+      if (valid) v = *reinterpret_cast<const pk::u32x4*>(qr + kk * 32);
+      qf[kk] = __builtin_bit_cast(pk::bf16x8_t, v);
+    }
+  }
+  pk::f32x4 o[NRT];
+#pragma unroll
+  for (int rt = 0; rt < NRT; ++rt) o[rt] = pk::f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+
+  for (int k0 = 0; k0 <= max_pos; k0 += BK) {
+    const int nk = min(BK, max_pos + 1 - k0);
+    for (int c = tid; c < BK * R8; c += 256) {
+      const int key = c / R8, r8 = c - key * R8;
+      pk::u32x4 v = {0u, 0u, 0u, 0u};
+      if (key < nk) {
+        const int kp = k0 + key;
+        const int64_t slot = static_cast<int64_t>(bt[kp / block_size]) * block_size + kp % block_size;
+        v = *reinterpret_cast<const pk::u32x4*>(cache + slot * R + r8 * 8);
+      }
+      *reinterpret_cast<pk::u32x4*>(cs + key * CS + r8 * 8) = v;
+      if (cache_t == nullptr) {  // no latent-major copy in the cache: transpose while staging
+        bf16_t* dst = ct + (r8 * 8) * CT + key_slot(key);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          dst[(2 * e) * CT] = static_cast<bf16_t>(v[e] & 0xffffu);
+          dst[(2 * e + 1) * CT] = static_cast<bf16_t>(v[e] >> 16);
+        }
+      }
+    }
+    if (cache_t) {  // the tile's latent-major copy is 64 contiguous bytes per latent coordinate
+      const bf16_t* src = cache_t + (static_cast<int64_t>(bt[k0 / block_size]) * (block_size / 32) +
+                                     (k0 % block_size) / 32) * R * 32;
+      for (int c = tid; c < R * 4; c += 256)
+        *reinterpret_cast<pk::u32x4*>(ct + (c >> 2) * CT + (c & 3) * 8) = *reinterpret_cast<const pk::u32x4*>(src + c * 8);
+    }
+    __syncthreads();
+    if (__any(my_pos >= k0)) {
+      pk::f32x4 sa[2] = {pk::f32x4{0.f, 0.f, 0.f, 0.f}, pk::f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        const bf16_t* kr = cs + (sub * 16 + n) * CS + 8 * g;
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk)
+          sa[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(kr + kk * 32), qf[kk], sa[sub], 0, 0, 0);
+      }
+      float sc[8];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = k0 + (e >> 2) * 16 + 4 * g + (e & 3);
+        sc[e] = key <= my_pos ? sa[e >> 2][e & 3] * scale : -INFINITY;
+        tmax = fmaxf(tmax, sc[e]);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m_run, tmax);
+      float p[8], tsum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p[e] = sc[e] == -INFINITY ? 0.f : expf(sc[e] - m_new);
+        tsum += p[e];
+      }
+      tsum += __shfl_xor(tsum, 16, 64);
+      tsum += __shfl_xor(tsum, 32, 64);
+      const float resc = m_run == -INFINITY ? (m_new == -INFINITY ? 1.f : 0.f) : expf(m_run - m_new);
+      m_run = m_new;
+      l_run = l_run * resc + tsum;
+      pk::u32x4 pw;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pw[e] = pk::pack2(p[2 * e], p[2 * e + 1]);
+      const pk::bf16x8_t pb = __builtin_bit_cast(pk::bf16x8_t, pw);
+      if (__any(resc != 1.f)) {
+#pragma unroll
+        for (int rt = 0; rt < NRT; ++rt) o[rt] *= resc;
+      }
+      const bf16_t* vr = ct + n * CT + 8 * g;
+#pragma unroll
+      for (int rt = 0; rt < NRT; ++rt)
+        o[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(vr + rt * 16 * CT), pb, o[rt], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  if (valid) {
+    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    bf16_t* dst = out + static_cast<int64_t>(q0 + tl) * out_st + static_cast<int64_t>(h) * out_sh + 4 * g;
+#pragma unroll
+    for (int rt = 0; rt < NRT; ++rt) {
+      uint2 w;
+      w.x = pk::pack2(o[rt][0] * inv, o[rt][1] * inv);
+      w.y = pk::pack2(o[rt][2] * inv, o[rt][3] * inv);
+      *reinterpret_cast<uint2*>(dst + rt * 16) = w;
+    }
+  }
+}
+
+// ---- decoding on the matrix cores -----------------------------------------------------------------
+// One query token per sequence: its H heads are the 16-row tiles.  Every wave owns a run of `part`
+// keys (a multiple of 32) and takes both products' A operands straight from the cache -- key-major
+// rows for S^T, the latent-major copy for O~^T -- so nothing is staged and no barrier is needed; it
+// leaves (max, sum, unnormalised o~) per head in the workspace and latent_merge_kernel combines the
+// runs.  `part` comes from the cache capacity, not from the batch: a position's sums are the same
+// in every step.
+template <int R>
+__global__ void __launch_bounds__(256)
+latent_decode_mfma_kernel(float* __restrict__ ws_o, float* __restrict__ ws_ml, const bf16_t* __restrict__ q,
+                          int64_t q_st, int64_t q_sh, const bf16_t* __restrict__ cache,
+                          const bf16_t* __restrict__ cache_t, const int* __restrict__ block_tables, int max_blocks,
+                          const int* __restrict__ cu_q, const int* __restrict__ context_lens, int H, int block_size,
+                          int part, int n_parts, float scale) {
+  constexpr int NKK = R / 32, NRT = R / 16;
+  const int s = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, n = lane & 15;
+  const int wp = blockIdx.y * 4 + wave;
+  const int ctx = context_lens[s], tok = cu_q[s];
+  const int k_lo = wp * part, k_hi = min(k_lo + part, ctx);
+  const int* bt = block_tables + static_cast<int64_t>(s) * max_blocks;
+  for (int h0 = 0; h0 < H; h0 += 16) {
+    const int h = h0 + n;
+    const bool valid = h < H;
+    const int64_t wrow = (static_cast<int64_t>(s) * n_parts + wp) * H + h;
+    if (k_lo >= k_hi) {  // an empty run
+      if (valid && g == 0) {
+        ws_ml[wrow * 2] = -INFINITY;
+        ws_ml[wrow * 2 + 1] = 0.f;
+      }
+      continue;
+    }
+    pk::bf16x8_t qf[NKK];
+    {
+      const bf16_t* qr = q + static_cast<int64_t>(tok) * q_st + static_cast<int64_t>(valid ? h : 0) * q_sh + 8 * g;
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        pk::u32x4 v = {0u, 0u, 0u, 0u};
+        if (valid) v = *reinterpret_cast<const pk::u32x4*>(qr + kk * 32);
+        qf[kk] = __builtin_bit_cast(pk::bf16x8_t, v);
+      }
+    }
+    pk::f32x4 o[NRT];
+#pragma unroll
+    for (int rt = 0; rt < NRT; ++rt) o[rt] = pk::f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
+      pk::f32x4 sa[2] = {pk::f32x4{0.f, 0.f, 0.f, 0.f}, pk::f32x4{0.f, 0.f, 0.f, 0.f}};
+      const int blk = bt[k0 / block_size];
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        const int kp = k0 + sub * 16 + n;  // this lane's key row; past the context: any cached row, masked below
+        const bf16_t* kr = cache + (static_cast<int64_t>(blk) * block_size + kp % block_size) * R + 8 * g;
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk)
+          sa[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(kr + kk * 32), qf[kk], sa[sub], 0, 0, 0);
+      }
+      float sc[8], tmax = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = k0 + (e >> 2) * 16 + 4 * g + (e & 3);
+        sc[e] = key < k_hi ? sa[e >> 2][e & 3] * scale : -INFINITY;
+        tmax = fmaxf(tmax, sc[e]);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m_run, tmax);
+      float p[8], tsum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p[e] = sc[e] == -INFINITY ? 0.f : expf(sc[e] - m_new);
+        tsum += p[e];
+      }
+      tsum += __shfl_xor(tsum, 16, 64);
+      tsum += __shfl_xor(tsum, 32, 64);
+      const float resc = m_run == -INFINITY ? 0.f : expf(m_run - m_new);
+      m_run = m_new;
+      l_run = l_run * resc + tsum;
+      pk::u32x4 pw;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pw[e] = pk::pack2(p[2 * e], p[2 * e + 1]);
+      const pk::bf16x8_t pb = __builtin_bit_cast(pk::bf16x8_t, pw);
+      if (__any(resc != 1.f)) {
+#pragma unroll
+        for (int rt = 0; rt < NRT; ++rt) o[rt] *= resc;
+      }
+      const bf16_t* vr = cache_t + ((static_cast<int64_t>(blk) * (block_size / 32) + (k0 % block_size) / 32) * R + n) * 32 + 8 * g;
+#pragma unroll
+      for (int rt = 0; rt < NRT; ++rt)
+        o[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(vr + rt * 16 * 32), pb, o[rt], 0, 0, 0);
+    }
+    if (valid) {
+      if (g == 0) {
+        ws_ml[wrow * 2] = m_run;
+        ws_ml[wrow * 2 + 1] = l_run;
+      }
+      float* dst = ws_o + wrow * R + 4 * g;
+#pragma unroll
+      for (int rt = 0; rt < NRT; ++rt) *reinterpret_cast<pk::f32x4*>(dst + rt * 16) = o[rt];
+    }
+  }
+}
+
+// out[token s, head h] = sum_p e^(m_p - M) o_p / sum_p e^(m_p - M) l_p over the n_parts runs
+__global__ void __launch_bounds__(128)
+latent_merge_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t out_sh, const float* __restrict__ ws_o,
+                    const float* __restrict__ ws_ml, const int* __restrict__ cu_q, int H, int R, int n_parts) {
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int64_t base = static_cast<int64_t>(s) * n_parts * H + h;
+  float M = -INFINITY;
+  for (int p = 0; p < n_parts; ++p) M = fmaxf(M, ws_ml[(base + static_cast<int64_t>(p) * H) * 2]);
+  float L = 0.f;
+  for (int p = 0; p < n_parts; ++p) {
+    const float m = ws_ml[(base + static_cast<int64_t>(p) * H) * 2];
+    if (m != -INFINITY) L += expf(m - M) * ws_ml[(base + static_cast<int64_t>(p) * H) * 2 + 1];
+  }
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  bf16_t* dst = out + static_cast<int64_t>(cu_q[s]) * out_st + static_cast<int64_t>(h) * out_sh;
+  for (int r = threadIdx.x; r < R; r += blockDim.x) {
+    float a = 0.f;
+    for (int p = 0; p < n_parts; ++p) {
+      const float m = ws_ml[(base + static_cast<int64_t>(p) * H) * 2];
+      if (m != -INFINITY) a += expf(m - M) * ws_o[(base + static_cast<int64_t>(p) * H) * R + r];
+    }
+    dst[r] = pk::f2bf(a * inv);
+  }
+}
+
+template <int R>
+static int launch_latent_decode(void* out, long long out_st, long long out_sh, const void* q, long long q_st,
+                                long long q_sh, const void* cache, const void* cache_t, const void* block_tables,
+                                int max_blocks, const void* cu_q, const void* context_lens, int n_seqs, int H,
+                                int block_size, float scale, void* ws_o, void* ws_ml, int part, int n_parts,
+                                hipStream_t stream) {
+  latent_decode_mfma_kernel<R><<<dim3(n_seqs, n_parts / 4), 256, 0, stream>>>(
+      static_cast<float*>(ws_o), static_cast<float*>(ws_ml), static_cast<const bf16_t*>(q), q_st, q_sh,
+      static_cast<const bf16_t*>(cache), static_cast<const bf16_t*>(cache_t), static_cast<const int*>(block_tables),
+      max_blocks, static_cast<const int*>(cu_q), static_cast<const int*>(context_lens), H, block_size, part, n_parts,
+      scale);
+  latent_merge_kernel<<<dim3(n_seqs, H), 128, 0, stream>>>(static_cast<bf16_t*>(out), out_st, out_sh,
+                                                           static_cast<const float*>(ws_o),
+                                                           static_cast<const float*>(ws_ml),
+                                                           static_cast<const int*>(cu_q), H, R, n_parts);
+  return PK_CHECK_LAUNCH();
+}
+
+template <int R>
+static int launch_latent_mfma(void* out, long long out_st, long long out_sh, const void* q, long long q_st,
+                              long long q_sh, const void* cache, const void* cache_t, const void* block_tables,
+                              int max_blocks, const void* cu_q, const void* context_lens, int n_seqs, int T, int H,
+                              int block_size, float scale, hipStream_t stream) {
+  constexpr size_t lds = (32 * (R + 8) + R * 40) * sizeof(bf16_t);
+  auto kern = latent_attention_mfma_kernel<R>;
+  if (lds > 48 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return static_cast<int>(e);
+  }
+  const int grid = static_cast<int>((static_cast<int64_t>(T) * H + 63) / 64 + n_seqs);
+  kern<<<grid, 256, lds, stream>>>(static_cast<bf16_t*>(out), out_st, out_sh, static_cast<const bf16_t*>(q), q_st, q_sh,
+                                   static_cast<const bf16_t*>(cache), static_cast<const bf16_t*>(cache_t),
+                                   static_cast<const int*>(block_tables), max_blocks, static_cast<const int*>(cu_q),
+                                   static_cast<const int*>(context_lens), n_seqs, H, block_size, scale);
+  return PK_CHECK_LAUNCH();
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 gate_merge_kernel(T* __restrict__ out, const T* __restrict__ o, int64_t o_st, int64_t o_sh, const T* __restrict__ g,
@@ -183,13 +505,22 @@ gate_merge_kernel(T* __restrict__ out, const T* __restrict__ o, int64_t o_st, in
 
 }  // namespace
 
-PK_EXPORT int pkm_latent_norm_cache(void* cache, const void* dkv, long long dkv_stride, const void* w,
-                                    const void* slot_mapping, int T, int R, float eps, int dt, hipStream_t stream) {
+PK_EXPORT int pkm_latent_norm_cache(void* cache, void* cache_t, int block_size, const void* dkv, long long dkv_stride,
+                                    const void* w, const void* slot_mapping, int T, int R, float eps, int dt,
+                                    hipStream_t stream) {
   if (T <= 0) return 0;
+  if (cache_t && (block_size <= 0 || block_size % 32)) return -1;
   PKM_DISPATCH(dt, E, latent_norm_cache_kernel<E><<<T, 128, 0, stream>>>(
-                          static_cast<E*>(cache), static_cast<const E*>(dkv), dkv_stride, static_cast<const float*>(w),
-                          static_cast<const int*>(slot_mapping), R, eps));
+                          static_cast<E*>(cache), static_cast<E*>(cache_t), block_size, static_cast<const E*>(dkv),
+                          dkv_stride, static_cast<const float*>(w), static_cast<const int*>(slot_mapping), R, eps));
   return PK_CHECK_LAUNCH();
+}
+
+// 0: every launch takes the fp32-FMA kernel (tests compare the two)
+static int g_latent_mfma = 1;
+PK_EXPORT int pkm_set_latent_mfma(int on) {
+  g_latent_mfma = on;
+  return 0;
 }
 
 // key tile size for a latent of R numbers: the largest of 64 / 32 / 16 / 8 whose tiles fit 96 KiB of LDS
@@ -201,11 +532,64 @@ static int latent_key_tile(int R) {
   return 0;
 }
 
+// latents the matrix-core kernels are built for
+PK_EXPORT int pkm_latent_mfma_rank(int R) {
+  switch (R) {
+    case 32: case 64: case 96: case 128: case 160: case 192: case 256: case 320: case 384: case 512:
+      return 1;
+    default:
+      return 0;
+  }
+}
+
+// Decoding: sequences 0..n_seqs-1 with ONE query token each (token cu_q[s]); bf16, a latent of
+// pkm_latent_mfma_rank, the latent-major cache copy.  ws_o [n_seqs, n_parts, H, R] and ws_ml
+// [n_seqs, n_parts, H, 2] fp32; `part` keys per run (multiple of 32), n_parts a multiple of 4 with
+// part * n_parts >= the longest context.
+PK_EXPORT int pkm_latent_decode(void* out, long long out_st, long long out_sh, const void* q, long long q_st,
+                                long long q_sh, const void* cache, const void* cache_t, const void* block_tables,
+                                int max_blocks, const void* cu_q, const void* context_lens, int n_seqs, int H, int R,
+                                int block_size, float scale, void* ws_o, void* ws_ml, int part, int n_parts,
+                                hipStream_t stream) {
+  if (n_seqs <= 0) return 0;
+  if (!cache_t || part <= 0 || part % 32 || n_parts <= 0 || n_parts % 4 || block_size % 32 || q_st % 8 || q_sh % 8 ||
+      reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(cache) % 16 ||
+      reinterpret_cast<uintptr_t>(cache_t) % 16)
+    return -1;
+#define PKM_LD(RR)                                                                                                  \
+  case RR:                                                                                                          \
+    return launch_latent_decode<RR>(out, out_st, out_sh, q, q_st, q_sh, cache, cache_t, block_tables, max_blocks,   \
+                                    cu_q, context_lens, n_seqs, H, block_size, scale, ws_o, ws_ml, part, n_parts,   \
+                                    stream);
+  switch (R) {
+    PKM_LD(32) PKM_LD(64) PKM_LD(96) PKM_LD(128) PKM_LD(160) PKM_LD(192) PKM_LD(256) PKM_LD(320) PKM_LD(384) PKM_LD(512)
+    default:
+      return -1;
+  }
+#undef PKM_LD
+}
+
 PK_EXPORT int pkm_latent_attention(void* out, long long out_st, long long out_sh, const void* q, long long q_st,
-                                   long long q_sh, const void* cache, const void* block_tables, int max_blocks,
-                                   const void* cu_q, const void* context_lens, int n_seqs, int T, int H, int R,
-                                   int block_size, float scale, int dt, hipStream_t stream) {
+                                   long long q_sh, const void* cache, const void* cache_t, const void* block_tables,
+                                   int max_blocks, const void* cu_q, const void* context_lens, int n_seqs, int T, int H,
+                                   int R, int block_size, float scale, int dt, hipStream_t stream) {
   if (T <= 0 || n_seqs <= 0) return 0;
+  if (cache_t && block_size % 32) return -1;
+  // bf16 with a latent the MFMA kernel is built for and 8-byte-aligned rows: the matrix cores
+  if (dt == kBF16 && g_latent_mfma && q_st % 8 == 0 && q_sh % 8 == 0 && out_st % 4 == 0 && out_sh % 4 == 0 &&
+      reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(cache) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out) % 8 == 0) {
+#define PKM_LM(RR)                                                                                                 \
+  case RR:                                                                                                         \
+    return launch_latent_mfma<RR>(out, out_st, out_sh, q, q_st, q_sh, cache, cache_t, block_tables, max_blocks,    \
+                                  cu_q, context_lens, n_seqs, T, H, block_size, scale, stream);
+    switch (R) {
+      PKM_LM(32) PKM_LM(64) PKM_LM(96) PKM_LM(128) PKM_LM(160) PKM_LM(192) PKM_LM(256) PKM_LM(320) PKM_LM(384) PKM_LM(512)
+      default:
+        break;
+    }
+#undef PKM_LM
+  }
   const int BK = latent_key_tile(R);
   if (BK == 0 || R > 1024 || block_size <= 0) return -1;
   const size_t lds = (static_cast<size_t>(kBQ + BK) * (R + 1) + kBQ * BK + 3 * kBQ) * sizeof(float);

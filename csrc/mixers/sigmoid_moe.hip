@@ -20,18 +20,33 @@ namespace {
 
 constexpr int kMaxTop = 16;
 
+// One wave per token.  WITH_DOT: the logits are computed here, z[e] = x . wr[e] (small batches:
+// one launch, a fixed summation order).  Otherwise `x` holds the fp32 logits [T, E] of a library
+// fp32 GEMM (large batches).  Then s = sigmoid(z) and `top` rounds of arg-max over the experts.
+template <bool WITH_DOT>
 __global__ void __launch_bounds__(64)
 route_sigmoid_topk_kernel(int* __restrict__ ids, float* __restrict__ wts, const float* __restrict__ x,
                           const float* __restrict__ wr, int W, int E, int top) {
   extern __shared__ float sc[];  // [E]
   const int t = blockIdx.x, lane = threadIdx.x;
-  const float* xr = x + static_cast<int64_t>(t) * W;
-  for (int e = 0; e < E; ++e) {
-    const float* w = wr + static_cast<int64_t>(e) * W;
-    float d = 0.f;
-    for (int i = lane; i < W; i += 64) d += xr[i] * w[i];
-    d = pk::wave_sum(d);
-    if (lane == 0) sc[e] = sigmoidf(d);
+  if (WITH_DOT) {
+    const float* xr = x + static_cast<int64_t>(t) * W;
+    for (int e = 0; e < E; ++e) {
+      const float* w = wr + static_cast<int64_t>(e) * W;
+      float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+      int i = lane;
+      for (; i + 192 < W; i += 256) {  // four independent loads in flight per lane
+        d0 += xr[i] * w[i];
+        d1 += xr[i + 64] * w[i + 64];
+        d2 += xr[i + 128] * w[i + 128];
+        d3 += xr[i + 192] * w[i + 192];
+      }
+      for (; i < W; i += 64) d0 += xr[i] * w[i];
+      const float d = pk::wave_sum((d0 + d1) + (d2 + d3));
+      if (lane == 0) sc[e] = sigmoidf(d);
+    }
+  } else {
+    for (int e = lane; e < E; e += 64) sc[e] = sigmoidf(x[static_cast<int64_t>(t) * E + e]);
   }
   __syncthreads();
   for (int k = 0; k < top; ++k) {
@@ -179,17 +194,32 @@ __global__ void __launch_bounds__(1024) expert_align_wide_kernel(const int* __re
   }
 }
 
-__global__ void __launch_bounds__(256) combine_rows_kernel(float* __restrict__ out, const float* __restrict__ y,
+template <typename Y>
+__global__ void __launch_bounds__(256) combine_rows_kernel(float* __restrict__ out, const Y* __restrict__ y,
                                                            const int* __restrict__ inv, int top, int W) {
   const int t = blockIdx.x;
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float a = 0.f;
     for (int k = 0; k < top; ++k) {
       const int r = inv[t * top + k];
-      if (r >= 0) a += y[static_cast<int64_t>(r) * W + i];
+      if (r >= 0) a += ld<Y>(y + static_cast<int64_t>(r) * W + i);
     }
     out[static_cast<int64_t>(t) * W + i] = a;
   }
+}
+
+// rows in expert order, each the fp32 stream row of its token times the slot's score: the input
+// of the framework's grouped expert GEMMs (the score scales the expert's input)
+template <typename T>
+__global__ void __launch_bounds__(256) permute_scaled_kernel(T* __restrict__ out, const float* __restrict__ x,
+                                                             const int* __restrict__ sorted_slots,
+                                                             const float* __restrict__ slot_scale, int top, int W) {
+  const int r = blockIdx.x;
+  const int slot = sorted_slots[r];
+  const float s = slot_scale[slot];
+  const float* src = x + static_cast<int64_t>(slot / top) * W;
+  T* dst = out + static_cast<int64_t>(r) * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) st<T>(dst + i, s * src[i]);
 }
 
 }  // namespace
@@ -198,9 +228,14 @@ PK_EXPORT int pkm_route_sigmoid_topk(void* ids, void* wts, const void* x, const 
                                      hipStream_t stream) {
   if (T <= 0) return 0;
   if (top < 1 || top > E || top > kMaxTop || E > 4096) return -1;
-  route_sigmoid_topk_kernel<<<T, 64, E * sizeof(float), stream>>>(static_cast<int*>(ids), static_cast<float*>(wts),
-                                                                  static_cast<const float*>(x),
-                                                                  static_cast<const float*>(wr), W, E, top);
+  // wr == nullptr: x holds the logits [T, E]
+  if (wr)
+    route_sigmoid_topk_kernel<true><<<T, 64, E * sizeof(float), stream>>>(
+        static_cast<int*>(ids), static_cast<float*>(wts), static_cast<const float*>(x), static_cast<const float*>(wr), W,
+        E, top);
+  else
+    route_sigmoid_topk_kernel<false><<<T, 64, E * sizeof(float), stream>>>(
+        static_cast<int*>(ids), static_cast<float*>(wts), static_cast<const float*>(x), nullptr, W, E, top);
   return PK_CHECK_LAUNCH();
 }
 
@@ -228,10 +263,21 @@ PK_EXPORT int pkm_expert_down(void* y, const void* h, const void* down, const vo
   return PK_CHECK_LAUNCH();
 }
 
-PK_EXPORT int pkm_combine_rows(void* out, const void* y, const void* inv, int T, int top, int W, hipStream_t stream) {
+// y_dt: element type of the expert outputs y
+PK_EXPORT int pkm_combine_rows(void* out, const void* y, const void* inv, int T, int top, int W, int y_dt,
+                               hipStream_t stream) {
   if (T <= 0) return 0;
-  combine_rows_kernel<<<T, 256, 0, stream>>>(static_cast<float*>(out), static_cast<const float*>(y),
-                                             static_cast<const int*>(inv), top, W);
+  PKM_DISPATCH(y_dt, Y, combine_rows_kernel<Y><<<T, 256, 0, stream>>>(static_cast<float*>(out), static_cast<const Y*>(y),
+                                                                      static_cast<const int*>(inv), top, W));
+  return PK_CHECK_LAUNCH();
+}
+
+PK_EXPORT int pkm_permute_scaled(void* out, const void* x, const void* sorted_slots, const void* slot_scale, int n,
+                                 int top, int W, int dt, hipStream_t stream) {
+  if (n <= 0) return 0;
+  PKM_DISPATCH(dt, T, permute_scaled_kernel<T><<<n, 256, 0, stream>>>(
+                          static_cast<T*>(out), static_cast<const float*>(x), static_cast<const int*>(sorted_slots),
+                          static_cast<const float*>(slot_scale), top, W));
   return PK_CHECK_LAUNCH();
 }
 

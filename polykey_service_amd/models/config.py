@@ -179,8 +179,14 @@ class SapapelConfig:
 ARCHITECTURES = {"Sapapel": SapapelConfig.from_json}
 
 PRESETS["tiny-sapapel"] = SapapelConfig.uniform("tiny-sapapel", 512, 128, 3, 4, 16, 32, 48, 64, 6, 2)
-# layer shapes of a ~1B-active latent-attention MoE (random weights; speed measurements)
-PRESETS["sapapel-2k"] = SapapelConfig.uniform("sapapel-2k", 32000, 2048, 8, 16, 128, 128, 512, 1408, 16, 2)
+# speed measurements (random weights): layer shapes of small production MoE models, and the
+# Mixtral-family model of the same width, depth, heads, experts and expert size beside each
+PRESETS["sapapel-2k"] = SapapelConfig.uniform("sapapel-2k", 32000, 2048, 8, 16, 128, 128, 512, 1536, 16, 2)
+PRESETS["sapapel-4k"] = SapapelConfig.uniform("sapapel-4k", 32000, 4096, 4, 32, 128, 128, 512, 2048, 8, 2)
+PRESETS["mixtral-2k"] = ModelConfig("mixtral-2k", 32000, 2048, 1536, 8, 16, 4, rope_theta=1e6, num_experts=16,
+                                    experts_per_token=2, bos_token_id=1, eos_token_id=2, router_init_std=0.5)
+PRESETS["mixtral-4k"] = ModelConfig("mixtral-4k", 32000, 4096, 2048, 4, 32, 8, rope_theta=1e6, num_experts=8,
+                                    experts_per_token=2, bos_token_id=1, eos_token_id=2, router_init_std=0.5)
 
 
 def get_config(name_or_path: str):

@@ -68,14 +68,16 @@ class LatentAttention(nn.Module):
         self.uv_t = _p(to(uv).view(H, V, R).transpose(1, 2))
         self.w_o = _p(to(o))
 
-    def forward(self, h: torch.Tensor, md, cache: torch.Tensor, eps: float) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, md, cache: torch.Tensor, eps: float,
+                cache_t: Optional[torch.Tensor] = None) -> torch.Tensor:
         s = self.spec
         H, D, V, R = s.heads, s.dim, s.vdim, s.kv_rank
         T = h.shape[0]
         qdg = gemm.linear(h, self.w_in)
-        la_ops.latent_norm_cache(qdg[:, H * D:H * D + R], self.latent_w, eps, cache, md.slot_mapping)
+        la_ops.latent_norm_cache(qdg[:, H * D:H * D + R], self.latent_w, eps, cache, md.slot_mapping, cache_t)
         q_lat = torch.bmm(qdg[:, :H * D].view(T, H, D).transpose(0, 1), self.uk)          # [H, T, R]
-        o_lat = la_ops.latent_attention(q_lat, cache, md.block_tables, md.cu_q, md.context_lens, md.num_seqs, s.scale)
+        o_lat = la_ops.latent_attention(q_lat, cache, md.block_tables, md.cu_q, md.context_lens, md.num_seqs, s.scale,
+                                        cache_t, md.num_decode)
         o = torch.bmm(o_lat, self.uv_t)                                                    # [H, T, V]
         return gemm.linear(la_ops.gate_merge(o, qdg[:, H * D + R:]), self.w_o)
 
@@ -87,14 +89,31 @@ class SigmoidMoE(nn.Module):
         self.router = None  # [E, W] fp32
         self.gate = self.up = self.down = None  # [E, F, W], [E, F, W], [E, W, F]
 
+        # shapes the grouped MFMA GEMMs tile: interleaved gate|up and down, block-packed for decode
+        self.w13 = self.w2 = self.w13_p = self.w2_p = None
+
     def set(self, router, gates, ups, downs, dtype, device) -> None:
         to = lambda ts: _p(torch.stack(ts).to(device=device, dtype=dtype))
         self.router = _p(router.to(device=device, dtype=torch.float32))
-        self.gate, self.up, self.down = to(gates), to(ups), to(downs)
+        E, (F_, W) = len(gates), gates[0].shape
+        if moe_ops.mfma_experts_ok(E, F_, W, dtype, torch.device(device)):
+            self.w13 = to([gemm.interleave_gate_up(g, u) for g, u in zip(gates, ups)])
+            self.w2 = to(downs)
+            self.gate = self.up = self.down = None
+        else:
+            self.gate, self.up, self.down = to(gates), to(ups), to(downs)
+
+    def pack(self) -> None:
+        if self.w13 is not None and self.w13_p is None:
+            E, N, K = self.w13.shape
+            self.w13_p = gemm.pack_weight(self.w13.view(E * N, K)).view(E, N, K)
+            E, N, K = self.w2.shape
+            self.w2_p = gemm.pack_weight(self.w2.view(E * N, K)).view(E, N, K)
 
     def forward(self, x: torch.Tensor, x_act: torch.Tensor) -> torch.Tensor:
         ids, wts = moe_ops.route_sigmoid_topk(x, self.router, self.spec.top)
-        return moe_ops.input_scaled_moe(x_act, ids, wts, self.gate, self.up, self.down)
+        return moe_ops.input_scaled_moe(x, x_act, ids, wts, self.gate, self.up, self.down, self.w13, self.w2,
+                                        self.w13_p, self.w2_p)
 
 
 class SapapelLayer(nn.Module):
@@ -140,7 +159,8 @@ class SapapelForCausalLM(nn.Module):
             L.g2 = f32(get(p + "norm2"))
             L.mlp.set(get(p + "mlp.router"), [get(p + f"mlp.e{e}.gate") for e in range(E)],
                       [get(p + f"mlp.e{e}.up") for e in range(E)], [get(p + f"mlp.e{e}.down") for e in range(E)], dt, dev)
-            assert L.mlp.gate.shape == (E, spec.mlp.ff, cfg.hidden_size)
+            got = L.mlp.gate.shape if L.mlp.gate is not None else (E, L.mlp.w13.shape[1] // 2, L.mlp.w13.shape[2])
+            assert tuple(got) == (E, spec.mlp.ff, cfg.hidden_size), (got, spec.mlp)
 
     def _set_top(self, get) -> None:
         dev, dt = self.device, self.dtype
@@ -168,8 +188,7 @@ class SapapelForCausalLM(nn.Module):
         """Random bf16-representable tensors under the checkpoint names (gains near 1, shift in
         [0, 1), depth weights near "mostly the newest output")."""
         cfg, W, std = self.cfg, self.cfg.hidden_size, self.cfg.init_std
-        cpu = torch.device("cpu")
-        r = lambda name, shape, s=std: random_full(name, shape, s, seed, cpu, torch.bfloat16)
+        r = lambda name, shape, s=std: random_full(name, shape, s, seed, self.device, torch.bfloat16)
         out = {"embed": r("embed", (cfg.vocab_size, W), 1.0), "head": r("head", (cfg.vocab_size, W)),
                "final.norm": 1 + r("final.norm", (), 0.1)}
         for i, l in enumerate(cfg.layers):
@@ -198,6 +217,12 @@ class SapapelForCausalLM(nn.Module):
     def init_random(self, seed: int = 0) -> "SapapelForCausalLM":
         return self.load_state(self.random_state(seed))
 
+    def pack_decode_weights(self) -> None:
+        """Block-packed copies of the expert weights for the decode GEMM (engine hook)."""
+        for L in self.layers:
+            if L.mlp is not None:
+                L.mlp.pack()
+
     def to(self, device, *a, **k):  # keeps the fp32 tensors fp32 (no dtype argument)
         super().to(device)
         self.device = torch.device(device)
@@ -207,16 +232,24 @@ class SapapelForCausalLM(nn.Module):
     # ---------------------------------------------------------- cache and state
     def cache_bytes_per_block(self, block_size: int) -> int:
         esz = 2 if self.dtype == torch.bfloat16 else 4
-        return sum(l.mixer.kv_rank for l in self.cfg.layers) * block_size * esz
+        copies = lambda R: 2 if la_ops.mfma_latent(R, self.dtype, self.device, block_size) else 1
+        return sum(l.mixer.kv_rank * copies(l.mixer.kv_rank) for l in self.cfg.layers) * block_size * esz
 
     def state_bytes_per_slot(self) -> int:
         return len(self.layers) * self.cfg.hidden_size * 4
 
     def alloc_cache(self, num_blocks: int, block_size: int, num_slots: int) -> List[tuple]:
-        """Per layer: (latent cache [blocks, block_size, kv_rank], shift state [slots, W] fp32)."""
-        return [(torch.zeros((num_blocks, block_size, l.mixer.kv_rank), dtype=self.dtype, device=self.device),
-                 torch.zeros((max(num_slots, 1), self.cfg.hidden_size), dtype=torch.float32, device=self.device))
-                for l in self.cfg.layers]
+        """Per layer: (latent cache [blocks, block_size, kv_rank], its latent-major copy for the
+        matrix-core kernels or None, shift state [slots, W] fp32)."""
+        out = []
+        for l in self.cfg.layers:
+            R = l.mixer.kv_rank
+            c = torch.zeros((num_blocks, block_size, R), dtype=self.dtype, device=self.device)
+            c_t = (la_ops.alloc_latent_major(num_blocks, block_size, R, self.device)
+                   if la_ops.mfma_latent(R, self.dtype, self.device, block_size) else None)
+            out.append((c, c_t, torch.zeros((max(num_slots, 1), self.cfg.hidden_size), dtype=torch.float32,
+                                            device=self.device)))
+        return out
 
     def activation_bytes_per_token(self) -> int:
         W = self.cfg.hidden_size
@@ -241,13 +274,13 @@ class SapapelForCausalLM(nn.Module):
         hist, eps, alpha, dt = self._hist, cfg.rms_eps, cfg.alpha, self.dtype
         x = stream_ops.embed_rows(self.embed, input_ids, hist[0])[:T]
         for i, L in enumerate(self.layers):
-            cache, state = caches[i]
+            cache, cache_t, state = caches[i]
             if L.shift is not None:
                 h = stream_ops.token_shift(x, L.shift, state, md.token_seq, md.cu_q, positions, md.state_slots, dt)
                 stream_ops.save_last_rows(x, state, md.cu_q, md.state_slots, md.num_seqs)
             else:
                 h = x.to(dt)
-            m = L.mix(h, md, cache, eps)
+            m = L.mix(h, md, cache, eps, cache_t)
             has_mlp = L.mlp is not None
             depth = dict(hist=hist, nh=i + 2, coef=L.dwa) if L.dwa is not None else {}
             out = torch.empty_like(x)

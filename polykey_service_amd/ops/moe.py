@@ -218,6 +218,12 @@ def fused_moe_reference(x, router_w, w13, w2, k, e_lo=0, e_hi=None):
 
 
 # ------------------------------------------------------------------ sigmoid-routed, input-scaled MoE
+# up to this many tokens the router's dot products run inside the top-k kernel; above, the logits
+# are one fp32 library GEMM.  0: always the GEMM (one wave per token walking every expert's row is
+# latency-bound: 173 us for 16 experts x 2048 against ~10 us for GEMM + top-k)
+ROUTER_DOT_MAX_T = 0
+
+
 def route_sigmoid_topk(x: torch.Tensor, router_w: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """fp32 router: s = sigmoid(router_w x); the k largest s per token and their experts (ties: the
     lower expert id), scores as they are.  x [T, W] fp32, router_w [E, W] fp32."""
@@ -230,20 +236,50 @@ def route_sigmoid_topk(x: torch.Tensor, router_w: torch.Tensor, k: int) -> Tuple
     assert x.dtype == torch.float32 and router_w.dtype == torch.float32 and x.is_contiguous()
     ids = torch.empty((T, k), dtype=torch.int32, device=x.device)
     w = torch.empty((T, k), dtype=torch.float32, device=x.device)
+    if T > ROUTER_DOT_MAX_T:  # many tokens: the logits as one fp32 library GEMM, then sigmoid + top-k
+        logits = torch.mm(x, router_w.t())
+        native.call("pkm_route_sigmoid_topk", ids.data_ptr(), w.data_ptr(), logits.data_ptr(), None, T, W, E, k,
+                    native.stream_ptr())
+        return ids, w
     native.call("pkm_route_sigmoid_topk", ids.data_ptr(), w.data_ptr(), x.data_ptr(), router_w.data_ptr(), T, W, E, k,
                 native.stream_ptr())
     return ids, w
 
 
-def input_scaled_moe(x_act: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
-                     down: torch.Tensor) -> torch.Tensor:
+def mfma_experts_ok(E: int, F_: int, W: int, dtype: torch.dtype, device) -> bool:
+    """Shapes the framework's MFMA grouped expert GEMMs tile (prefill: 256-wide column tiles; decode:
+    the weight-streaming grouped GEMM on block-packed experts): bf16 on the GPU, at most 64 experts,
+    ff and width multiples of 256."""
+    return (device.type == "cuda" and dtype == torch.bfloat16 and E <= 64 and F_ % 256 == 0 and W % 256 == 0)
+
+
+def input_scaled_moe(x: torch.Tensor, x_act: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, gate, up, down,
+                     w13=None, w2=None, w13_p=None, w2_p=None) -> torch.Tensor:
     """sum over a token's experts of down_e(silu(gate_e(s x)) * up_e(s x)), s the expert's score,
-    as fp32 [T, W].  x_act [T, W] in the weights' dtype; gate / up [E, F, W]; down [E, W, F].
-    Tokens are grouped by expert on the device (align), the score is applied to the gate / up
-    products, and the combine is a plain sum."""
+    as fp32 [T, W].  x: the fp32 stream rows, x_act: the same in the weights' dtype.  Tokens are
+    grouped by expert on the device (align) and the combine is a plain sum.
+
+    Two forms.  With ``w13`` / ``w2`` (interleaved gate|up [E, 2F, W] and down [E, W, F], shapes of
+    :func:`mfma_experts_ok`): rows ``s * x`` in expert order feed the framework's grouped MFMA
+    GEMMs with the fused SiLU epilogue.  Otherwise (any sizes, fp32): gate / up [E, F, W] and down
+    [E, W, F] through the tiled fp32-FMA grouped kernels, the score applied to the gate / up
+    products (the same value, the products' accumulations left unscaled)."""
     T, W = x_act.shape
-    E, F_, _ = gate.shape
     k = ids.shape[1]
+    n = T * k
+    if w13 is not None:
+        E = w13.shape[0]
+        offsets, sorted_, inv = align(ids, E, 0, E)
+        st = native.stream_ptr()
+        xs = torch.empty((n, W), dtype=x_act.dtype, device=x.device)
+        native.call("pkm_permute_scaled", xs.data_ptr(), x.data_ptr(), sorted_.data_ptr(), wts.data_ptr(), n, k, W,
+                    native.dt_code(xs.dtype), st)
+        h = grouped_gemm(xs, w13, offsets, T, silu=True, packed=w13_p)
+        y = grouped_gemm(h, w2, offsets, T, silu=False, packed=w2_p)
+        out = torch.empty((T, W), dtype=torch.float32, device=x.device)
+        native.call("pkm_combine_rows", out.data_ptr(), y.data_ptr(), inv.data_ptr(), T, k, W, native.dt_code(y.dtype), st)
+        return out
+    E, F_, _ = gate.shape
     offsets, sorted_, inv = align(ids, E, 0, E)
     if not x_act.is_cuda:
         m = int(offsets[-1])
@@ -263,7 +299,6 @@ def input_scaled_moe(x_act: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, 
     assert x_act.is_contiguous() and gate.is_contiguous() and up.is_contiguous() and down.is_contiguous()
     assert gate.dtype == x_act.dtype and wts.dtype == torch.float32 and wts.is_contiguous()
     dt = native.dt_code(x_act.dtype)
-    n = T * k
     h = torch.empty((n, F_), dtype=x_act.dtype, device=x_act.device)
     y = torch.empty((n, W), dtype=torch.float32, device=x_act.device)
     out = torch.empty((T, W), dtype=torch.float32, device=x_act.device)
@@ -271,5 +306,5 @@ def input_scaled_moe(x_act: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, 
     native.call("pkm_expert_gate_up", h.data_ptr(), x_act.data_ptr(), gate.data_ptr(), up.data_ptr(), offsets.data_ptr(),
                 sorted_.data_ptr(), wts.data_ptr(), n, k, E, F_, W, dt, st)
     native.call("pkm_expert_down", y.data_ptr(), h.data_ptr(), down.data_ptr(), offsets.data_ptr(), n, E, W, F_, dt, st)
-    native.call("pkm_combine_rows", out.data_ptr(), y.data_ptr(), inv.data_ptr(), T, k, W, st)
+    native.call("pkm_combine_rows", out.data_ptr(), y.data_ptr(), inv.data_ptr(), T, k, W, 1, st)
     return out

@@ -73,13 +73,17 @@ MIXER_SIGNATURES = {
     "pkm_token_shift": [P, P, P, P, P, P, P, P, I32, I32, I32, P],
     "pkm_save_last_rows": [P, P, P, P, I32, I32, P],
     "pkm_sum_gain_norm": [P, P, P, P, P, F32, P, F32, I32, I32, P, I64, I32, P, I32, I32, P],
-    "pkm_latent_norm_cache": [P, P, I64, P, P, I32, I32, F32, I32, P],
-    "pkm_latent_attention": [P, I64, I64, P, I64, I64, P, P, I32, P, P, I32, I32, I32, I32, I32, F32, I32, P],
+    "pkm_latent_norm_cache": [P, P, I32, P, I64, P, P, I32, I32, F32, I32, P],
+    "pkm_latent_attention": [P, I64, I64, P, I64, I64, P, P, P, I32, P, P, I32, I32, I32, I32, I32, F32, I32, P],
+    "pkm_latent_decode": [P, I64, I64, P, I64, I64, P, P, P, I32, P, P, I32, I32, I32, I32, F32, P, P, I32, I32, P],
+    "pkm_latent_mfma_rank": [I32],
+    "pkm_set_latent_mfma": [I32],
     "pkm_gate_merge": [P, P, I64, I64, P, I64, I32, I32, I32, I32, P],
     "pkm_route_sigmoid_topk": [P, P, P, P, I32, I32, I32, I32, P],
     "pkm_expert_gate_up": [P, P, P, P, P, P, P, I32, I32, I32, I32, I32, I32, P],
     "pkm_expert_down": [P, P, P, P, I32, I32, I32, I32, I32, P],
-    "pkm_combine_rows": [P, P, P, I32, I32, I32, P],
+    "pkm_combine_rows": [P, P, P, I32, I32, I32, I32, P],
+    "pkm_permute_scaled": [P, P, P, P, I32, I32, I32, I32, P],
     "pkm_expert_align_wide": [P, P, P, P, I32, I32, P],
 }
 _mixers: Optional[ctypes.CDLL] = None

@@ -129,6 +129,99 @@ def test_sigmoid_moe(dt, E, k, F, W, T):
     torch.testing.assert_close(w_g.cpu(), w_c, rtol=1e-5, atol=1e-6)
     gate, up, down = (torch.randn(E, F, W) * 0.2).to(dt), (torch.randn(E, F, W) * 0.2).to(dt), (torch.randn(E, W, F) * 0.2).to(dt)
     xa = x.to(dt)
-    want = moe.input_scaled_moe(xa, ids_c, w_c, gate, up, down)
-    got = moe.input_scaled_moe(xa.to(dev), ids_g, w_g, gate.to(dev), up.to(dev), down.to(dev))
+    want = moe.input_scaled_moe(x, xa, ids_c, w_c, gate, up, down)
+    got = moe.input_scaled_moe(x.to(dev), xa.to(dev), ids_g, w_g, gate.to(dev), up.to(dev), down.to(dev))
     torch.testing.assert_close(got.cpu(), want, **(dict(rtol=1e-4, atol=1e-4) if dt == torch.float32 else tol(dt)))
+
+
+def latent_major(cache):
+    """[blocks, bs, R] -> [blocks, bs / 32, R, 32] with key k of a 32-key tile in column
+    8 * ((k % 16) // 4) + k % 4 + 4 * (k // 16)."""
+    nb, bs, R = cache.shape
+    k = torch.arange(32)
+    col = 8 * ((k % 16) // 4) + k % 4 + 4 * (k // 16)
+    out = torch.zeros(nb, bs // 32, R, 32, dtype=cache.dtype)
+    out[:, :, :, col] = cache.view(nb, bs // 32, 32, R).transpose(2, 3)
+    return out
+
+
+@pytest.mark.parametrize("H,R", [(8, 96), (16, 128), (5, 512), (3, 32), (20, 64)])
+def test_latent_attention_matrix_core_kernels(H, R):
+    """bf16 latents the MFMA kernels are built for: against the fp32 composition and against the
+    FMA kernel on the same inputs; decoded tokens (decode kernel, runs merged) beside prompt
+    portions over several row tiles, with and without the latent-major cache copy."""
+    from polykey_service_amd.ops import native
+    dev, bs = torch.device("cuda"), 32
+    qlens, ctxs = [1, 1, 1, 70, 9, 33], [300, 31, 64, 70, 140, 97]
+    m = batch_meta(qlens, ctxs, bs, torch.device("cpu"))
+    T = sum(qlens)
+    cache = (torch.randn(m["nblocks"], bs, R) * 0.7).bfloat16()
+    q = (torch.randn(H, T, R) * 0.4).bfloat16()
+    want = la.latent_attention(q, cache, m["bt"], m["cu_q"], m["ctx"], 6, R ** -0.5).float()
+    args = (q.to(dev), cache.to(dev), m["bt"].to(dev), m["cu_q"].to(dev), m["ctx"].to(dev), 6, R ** -0.5)
+    got = la.latent_attention(*args)
+    got_t = la.latent_attention(*args, latent_major(cache).to(dev), 3)
+    native.call("pkm_set_latent_mfma", 0)
+    try:
+        fma = la.latent_attention(*args)
+    finally:
+        native.call("pkm_set_latent_mfma", 1)
+    for x in (fma, got, got_t):
+        torch.testing.assert_close(x.cpu().float(), want, rtol=2e-2, atol=1e-2)
+    assert not torch.equal(got, fma) or R == 32  # two kernels ran
+    assert la.mfma_latent(R, torch.bfloat16, dev, bs) and not la.mfma_latent(R + 8, torch.bfloat16, dev, bs)
+
+
+def test_norm_cache_writes_both_layouts():
+    dev, bs, R = torch.device("cuda"), 64, 96
+    m = batch_meta([70, 1], [70, 130], bs, torch.device("cpu"))
+    dkv = torch.randn(71, R).bfloat16()
+    w = 1 + 0.1 * torch.randn(R)
+    c = torch.zeros(m["nblocks"], bs, R, dtype=torch.bfloat16, device=dev)
+    c_t = la.alloc_latent_major(m["nblocks"], bs, R, dev)
+    la.latent_norm_cache(dkv.to(dev), w.to(dev), 1e-5, c, m["slots"].to(dev), c_t)
+    assert torch.equal(c_t.cpu(), latent_major(c.cpu())) and float(c.float().abs().sum()) > 0
+
+
+@pytest.mark.parametrize("key", [0, 31, 32, 63, 64, 65, 500, 991])
+def test_decode_kernel_finds_one_far_key(key):
+    """A decoded token whose query matches ONE cached key (first key, either side of a page border,
+    either side of a run border of the split context, the newest key): the output is that latent."""
+    dev, bs, R, ctx = torch.device("cuda"), 32, 64, 992
+    assert la.decode_runs(1024)[0] == 64  # keys 63 | 64 sit on a run border
+    m = batch_meta([1], [ctx], bs, torch.device("cpu"))
+    c = torch.randn(ctx, R) * 0.1
+    c[key] = c[key] / c[key].norm() * 4.0
+    q = (30.0 * c[key] / c[key].norm()).view(1, 1, R).repeat(3, 1, 1).bfloat16()
+    cache = torch.zeros(m["nblocks"], bs, R)
+    idx = torch.arange(ctx)
+    cache.view(-1, R)[m["bt"][0].long()[idx // bs] * bs + idx % bs] = c
+    cache = cache.bfloat16()
+    out = la.latent_attention(q.to(dev), cache.to(dev), m["bt"].to(dev), m["cu_q"].to(dev), m["ctx"].to(dev), 1, 1.0,
+                              latent_major(cache).to(dev), 1)
+    torch.testing.assert_close(out[1, 0].cpu().float(), c[key].bfloat16().float(), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("E,k,F,W,T", [(4, 2, 256, 256, 40), (8, 1, 512, 256, 300)])
+def test_sigmoid_moe_on_grouped_mfma_gemms(E, k, F, W, T):
+    """Shapes the framework's grouped MFMA expert GEMMs tile: rows scaled by their score, then the
+    interleaved gate|up GEMM with the SiLU epilogue and the down GEMM, against the fp32 composition."""
+    from polykey_service_amd.ops import gemm
+    dev = torch.device("cuda")
+    assert moe.mfma_experts_ok(E, F, W, torch.bfloat16, dev)
+    x = torch.randn(T, W)
+    rw = torch.randn(E, W) * 0.3
+    ids, wts = moe.route_sigmoid_topk(x, rw, k)
+    gate, up, down = ((torch.randn(E, F, W) * 0.1).bfloat16(), (torch.randn(E, F, W) * 0.1).bfloat16(),
+                      (torch.randn(E, W, F) * 0.1).bfloat16())
+    want = moe.input_scaled_moe(x, x.bfloat16(), ids, wts, gate, up, down)
+    w13 = torch.stack([gemm.interleave_gate_up(gate[e], up[e]) for e in range(E)]).to(dev)
+    w2 = down.to(dev)
+    for packed in (False, True):
+        w13_p = gemm.pack_weight(w13.view(E * 2 * F, W)).view(E, 2 * F, W) if packed else None
+        w2_p = gemm.pack_weight(w2.view(E * W, F)).view(E, W, F) if packed else None
+        got = moe.input_scaled_moe(x.to(dev), x.bfloat16().to(dev), ids.to(dev), wts.to(dev), None, None, None, w13, w2,
+                                   w13_p, w2_p)
+        err = (got.cpu() - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()
+        assert float(err) < 1e-2, float(err)  # bf16 rounding of the scaled rows, h and y
+        assert float((got.cpu() - want).abs().max()) < 0.05 * float(want.abs().max())

@@ -135,7 +135,7 @@ def test_latent_attention_mixer(device, H, D, V, R):
     for a, b in ((0, 31), (31, 33), (33, 34), (34, 70)):  # portions across the page borders at 32 and 64
         pos = torch.arange(a, b)
         md = AttnMetadata(0, 1, b - a, b - a, (table[0].cpu()[pos // BS] * BS + pos % BS).to(torch.int32).to(dev))
-        md.num_seqs, md.block_tables = 1, table
+        md.num_seqs, md.block_tables, md.num_decode = 1, table, 0
         md.cu_q = torch.tensor([0, b - a], dtype=torch.int32, device=dev)
         md.context_lens = torch.tensor([b], dtype=torch.int32, device=dev)
         got.append(mix(h[a:b].to(dev), md, cache, 1e-5).cpu())
