@@ -427,28 +427,33 @@ latent_decode_mfma_kernel(float* __restrict__ ws_o, float* __restrict__ ws_ml, c
   }
 }
 
-// out[token s, head h] = sum_p e^(m_p - M) o_p / sum_p e^(m_p - M) l_p over the n_parts runs
+// out[token s, head h] = sum_p e^(m_p - M) o_p / sum_p e^(m_p - M) l_p over the n_parts (<= 64) runs:
+// the first wave turns the runs' (max, sum) into weights, then every thread sums its coordinates
 __global__ void __launch_bounds__(128)
 latent_merge_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t out_sh, const float* __restrict__ ws_o,
                     const float* __restrict__ ws_ml, const int* __restrict__ cu_q, int H, int R, int n_parts) {
+  __shared__ float wgt[64];
   const int s = blockIdx.x, h = blockIdx.y;
   const int64_t base = static_cast<int64_t>(s) * n_parts * H + h;
-  float M = -INFINITY;
-  for (int p = 0; p < n_parts; ++p) M = fmaxf(M, ws_ml[(base + static_cast<int64_t>(p) * H) * 2]);
-  float L = 0.f;
-  for (int p = 0; p < n_parts; ++p) {
-    const float m = ws_ml[(base + static_cast<int64_t>(p) * H) * 2];
-    if (m != -INFINITY) L += expf(m - M) * ws_ml[(base + static_cast<int64_t>(p) * H) * 2 + 1];
+  if (threadIdx.x < 64) {
+    const int p = threadIdx.x;
+    const bool in = p < n_parts;
+    const float m = in ? ws_ml[(base + static_cast<int64_t>(p) * H) * 2] : -INFINITY;
+    const float l = in ? ws_ml[(base + static_cast<int64_t>(p) * H) * 2 + 1] : 0.f;
+    const float M = pk::wave_max(m);
+    const float w = m == -INFINITY ? 0.f : expf(m - M);
+    const float L = pk::wave_sum(w * l);
+    wgt[p] = L > 0.f ? w / L : 0.f;
   }
-  const float inv = L > 0.f ? 1.f / L : 0.f;
+  __syncthreads();
   bf16_t* dst = out + static_cast<int64_t>(cu_q[s]) * out_st + static_cast<int64_t>(h) * out_sh;
   for (int r = threadIdx.x; r < R; r += blockDim.x) {
     float a = 0.f;
     for (int p = 0; p < n_parts; ++p) {
-      const float m = ws_ml[(base + static_cast<int64_t>(p) * H) * 2];
-      if (m != -INFINITY) a += expf(m - M) * ws_o[(base + static_cast<int64_t>(p) * H) * R + r];
+      const float w = wgt[p];
+      if (w != 0.f) a += w * ws_o[(base + static_cast<int64_t>(p) * H) * R + r];
     }
-    dst[r] = pk::f2bf(a * inv);
+    dst[r] = pk::f2bf(a);
   }
 }
 
@@ -552,7 +557,7 @@ PK_EXPORT int pkm_latent_decode(void* out, long long out_st, long long out_sh, c
                                 int block_size, float scale, void* ws_o, void* ws_ml, int part, int n_parts,
                                 hipStream_t stream) {
   if (n_seqs <= 0) return 0;
-  if (!cache_t || part <= 0 || part % 32 || n_parts <= 0 || n_parts % 4 || block_size % 32 || q_st % 8 || q_sh % 8 ||
+  if (!cache_t || part <= 0 || part % 32 || n_parts <= 0 || n_parts % 4 || n_parts > 64 || block_size % 32 || q_st % 8 || q_sh % 8 ||
       reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(cache) % 16 ||
       reinterpret_cast<uintptr_t>(cache_t) % 16)
     return -1;

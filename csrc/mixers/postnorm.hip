@@ -63,26 +63,57 @@ __global__ void __launch_bounds__(256) save_last_rows_kernel(float* __restrict__
   for (int i = threadIdx.x; i < W; i += blockDim.x) dst[i] = src[i];
 }
 
+// Optional fused neighbours:
+//   gather (inv, top):  y is a table of expert output rows and the token's y is the plain sum of its
+//                       `top` rows y[inv[t * top + j]] (the MoE combine; inv < 0: no row)
+//   state (token_seq, cu_q, slots): a token that is the last of its sequence in this step leaves its
+//                       x row in the sequence's state slot (the token shift of the NEXT step reads it;
+//                       this step's shift has already run)
+struct NormFusion {
+  const int* inv;
+  int top;
+  float* state;
+  const int* token_seq;
+  const int* cu_q;
+  const int* slots;
+};
+
 template <typename T, typename Y>
 __global__ void __launch_bounds__(256)
 sum_gain_norm_kernel(float* __restrict__ out, T* __restrict__ out_act, const float* __restrict__ x,
                      const Y* __restrict__ y, const int* __restrict__ rows, float alpha, const float* __restrict__ gain,
                      float eps, int W, float* __restrict__ hist, int64_t hist_stride, int nh,
-                     const float* __restrict__ coef) {
+                     const float* __restrict__ coef, NormFusion f) {
   __shared__ float red[16];
+  extern __shared__ float vbuf[];  // [W] the sum alpha x + y, kept between the two passes
   const int r = blockIdx.x;
   const int64_t src = rows ? rows[r] : r;
   const float* xr = x + src * W;
-  const Y* yr = y ? y + src * W : nullptr;
+  const Y* yr = (y && !f.inv) ? y + src * W : nullptr;
+  float* keep = nullptr;
+  if (f.state) {
+    const int sq = f.token_seq[r];
+    if (r == f.cu_q[sq + 1] - 1 && f.slots[sq] >= 0) keep = f.state + static_cast<int64_t>(f.slots[sq]) * W;
+  }
   float ss = 0.f;
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    const float v = alpha * xr[i] + (yr ? ld<Y>(yr + i) : 0.f);
+    const float xv = xr[i];
+    float yv = yr ? ld<Y>(yr + i) : 0.f;
+    if (f.inv) {
+      for (int j = 0; j < f.top; ++j) {
+        const int yrow = f.inv[src * f.top + j];
+        if (yrow >= 0) yv += ld<Y>(y + static_cast<int64_t>(yrow) * W + i);
+      }
+    }
+    if (keep) keep[i] = xv;
+    const float v = alpha * xv + yv;
+    vbuf[i] = v;
     ss += v * v;
   }
   ss = pk::block_sum(ss, red);
   const float k = gain[0] / sqrtf(ss / static_cast<float>(W) + eps);
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    float z = (alpha * xr[i] + (yr ? ld<Y>(yr + i) : 0.f)) * k;
+    float z = vbuf[i] * k;
     if (hist) {
       const int64_t at = static_cast<int64_t>(r) * W + i;
       hist[(nh - 1) * hist_stride + at] = z;
@@ -125,19 +156,26 @@ PK_EXPORT int pkm_save_last_rows(void* state, const void* x, const void* cu_q, c
   return PK_CHECK_LAUNCH();
 }
 
-// y_dt: element type of y (-1: no y).  hist == nullptr: no history / average.
+// y_dt: element type of y (-1: no y).  hist == nullptr: no history / average.  inv != nullptr: y is
+// gathered (see NormFusion); state != nullptr: last rows are saved (token_seq, cu_q, slots given).
 PK_EXPORT int pkm_sum_gain_norm(void* out, void* out_act, const void* x, const void* y, const void* rows, float alpha,
                                 const void* gain, float eps, int R, int W, void* hist, long long hist_stride, int nh,
-                                const void* coef, int dt, int y_dt, hipStream_t stream) {
+                                const void* coef, int dt, int y_dt, const void* inv, int top, void* state,
+                                const void* token_seq, const void* cu_q, const void* slots, hipStream_t stream) {
   if (R <= 0) return 0;
   if (hist && (nh < 1 || !coef)) return -1;
+  if ((inv && (!y || top < 1 || rows)) || (state && (!token_seq || !cu_q || !slots || rows))) return -1;
+  if (W > 16384) return -1;
+  const NormFusion f{static_cast<const int*>(inv), top, static_cast<float*>(state), static_cast<const int*>(token_seq),
+                     static_cast<const int*>(cu_q), static_cast<const int*>(slots)};
+  const size_t lds = static_cast<size_t>(W) * sizeof(float);
 #define PKM_SGN(E, Y)                                                                                             \
-  sum_gain_norm_kernel<E, Y><<<R, 256, 0, stream>>>(static_cast<float*>(out), static_cast<E*>(out_act),           \
-                                                    static_cast<const float*>(x), static_cast<const Y*>(y),       \
-                                                    static_cast<const int*>(rows), alpha,                         \
-                                                    static_cast<const float*>(gain), eps, W,                      \
-                                                    static_cast<float*>(hist), hist_stride, nh,                   \
-                                                    static_cast<const float*>(coef))
+  sum_gain_norm_kernel<E, Y><<<R, 256, lds, stream>>>(static_cast<float*>(out), static_cast<E*>(out_act),         \
+                                                      static_cast<const float*>(x), static_cast<const Y*>(y),     \
+                                                      static_cast<const int*>(rows), alpha,                       \
+                                                      static_cast<const float*>(gain), eps, W,                    \
+                                                      static_cast<float*>(hist), hist_stride, nh,                 \
+                                                      static_cast<const float*>(coef), f)
   if (y == nullptr || y_dt == kF32) {
     PKM_DISPATCH(dt, E, PKM_SGN(E, float));
   } else if (y_dt == kBF16) {

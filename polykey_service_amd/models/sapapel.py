@@ -13,10 +13,12 @@ dtype, bf16 or fp32; every norm, the stream, scores, the router and the state ar
     o~     = softmax(scale q~ C^T) C           causal, over the cached latents           HIP  latent_attention.hip
     o      = o~[a] @ Wuv[a]^T per head         values out of the latent space            hipBLASLt (batched)
     m      = (o * sigmoid(g)) @ Wo^T           output gate + projection                  HIP gate_merge + GEMM
-    x1     = norm(alpha x + m) * g1            one-number gain                           HIP  postnorm.hip
+    x1     = norm(alpha x + m) * g1            one-number gain; also leaves x in the     HIP  postnorm.hip
+                                               sequences' state slots
     ids, s = top-k of sigmoid(Wr x1)           fp32 router                               HIP  sigmoid_moe.hip
     f      = sum_e down_e(silu(s gate_e x1) * (s up_e x1))                                HIP  sigmoid_moe.hip
     X[i+1] = norm(alpha x1 + f) * g2 ;  x' = sum_j dwa_i[j] X[j]     (X[0] = the embedding)  HIP  postnorm.hip
+             (one kernel: the experts' rows are summed, normed and averaged over depth)
 
 and logits = head @ (norm(x_last) * g_final).  Only c is cached (kv_rank numbers per token and
 layer); the per-sequence state is one stream row per layer.  Tensor parallelism is not
@@ -110,10 +112,12 @@ class SigmoidMoE(nn.Module):
             E, N, K = self.w2.shape
             self.w2_p = gemm.pack_weight(self.w2.view(E * N, K)).view(E, N, K)
 
-    def forward(self, x: torch.Tensor, x_act: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, x_act: torch.Tensor, defer_combine: bool = False):
+        """The experts' summed output [T, W] fp32, or with ``defer_combine`` the expert rows and their
+        inverse positions for the following norm kernel to sum."""
         ids, wts = moe_ops.route_sigmoid_topk(x, self.router, self.spec.top)
         return moe_ops.input_scaled_moe(x, x_act, ids, wts, self.gate, self.up, self.down, self.w13, self.w2,
-                                        self.w13_p, self.w2_p)
+                                        self.w13_p, self.w2_p, defer_combine)
 
 
 class SapapelLayer(nn.Module):
@@ -275,9 +279,10 @@ class SapapelForCausalLM(nn.Module):
         x = stream_ops.embed_rows(self.embed, input_ids, hist[0])[:T]
         for i, L in enumerate(self.layers):
             cache, cache_t, state = caches[i]
+            save = None
             if L.shift is not None:
                 h = stream_ops.token_shift(x, L.shift, state, md.token_seq, md.cu_q, positions, md.state_slots, dt)
-                stream_ops.save_last_rows(x, state, md.cu_q, md.state_slots, md.num_seqs)
+                save = (state, md.token_seq, md.cu_q, md.state_slots)  # the first norm kernel leaves x there
             else:
                 h = x.to(dt)
             m = L.mix(h, md, cache, eps, cache_t)
@@ -285,11 +290,12 @@ class SapapelForCausalLM(nn.Module):
             depth = dict(hist=hist, nh=i + 2, coef=L.dwa) if L.dwa is not None else {}
             out = torch.empty_like(x)
             if has_mlp:
-                x1, x1_act = stream_ops.sum_gain_norm(x, m, alpha, L.g1, eps, out=torch.empty_like(x), act_dtype=dt)
-                f = L.mlp(x1, x1_act)
-                x, _ = stream_ops.sum_gain_norm(x1, f, alpha, L.g2, eps, out=out, **depth)
+                x1, x1_act = stream_ops.sum_gain_norm(x, m, alpha, L.g1, eps, out=torch.empty_like(x), act_dtype=dt,
+                                                      save=save)
+                y, inv = L.mlp(x1, x1_act, defer_combine=True)
+                x, _ = stream_ops.sum_gain_norm(x1, y, alpha, L.g2, eps, out=out, gather=(inv, L.mlp.spec.top), **depth)
             else:
-                x, _ = stream_ops.sum_gain_norm(x, m, alpha, L.g1, eps, out=out, **depth)
+                x, _ = stream_ops.sum_gain_norm(x, m, alpha, L.g1, eps, out=out, save=save, **depth)
             if L.dwa is None:  # later layers' averages still read this layer's output
                 hist[i + 1, :T] = x
         return x

@@ -254,10 +254,12 @@ def mfma_experts_ok(E: int, F_: int, W: int, dtype: torch.dtype, device) -> bool
 
 
 def input_scaled_moe(x: torch.Tensor, x_act: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, gate, up, down,
-                     w13=None, w2=None, w13_p=None, w2_p=None) -> torch.Tensor:
+                     w13=None, w2=None, w13_p=None, w2_p=None, defer_combine: bool = False):
     """sum over a token's experts of down_e(silu(gate_e(s x)) * up_e(s x)), s the expert's score,
     as fp32 [T, W].  x: the fp32 stream rows, x_act: the same in the weights' dtype.  Tokens are
-    grouped by expert on the device (align) and the combine is a plain sum.
+    grouped by expert on the device (align) and the combine is a plain sum; with ``defer_combine``
+    the expert rows and their inverse positions (y [T * top, W], inv [T * top]) are returned for
+    the norm kernel that follows to sum (stream.sum_gain_norm ``gather``).
 
     Two forms.  With ``w13`` / ``w2`` (interleaved gate|up [E, 2F, W] and down [E, W, F], shapes of
     :func:`mfma_experts_ok`): rows ``s * x`` in expert order feed the framework's grouped MFMA
@@ -276,6 +278,8 @@ def input_scaled_moe(x: torch.Tensor, x_act: torch.Tensor, ids: torch.Tensor, wt
                     native.dt_code(xs.dtype), st)
         h = grouped_gemm(xs, w13, offsets, T, silu=True, packed=w13_p)
         y = grouped_gemm(h, w2, offsets, T, silu=False, packed=w2_p)
+        if defer_combine:
+            return y, inv
         out = torch.empty((T, W), dtype=torch.float32, device=x.device)
         native.call("pkm_combine_rows", out.data_ptr(), y.data_ptr(), inv.data_ptr(), T, k, W, native.dt_code(y.dtype), st)
         return out
@@ -295,6 +299,8 @@ def input_scaled_moe(x: torch.Tensor, x_act: torch.Tensor, ids: torch.Tensor, wt
                 u = (xe @ up[e].float().t()) * s[lo:hi, None]
                 h = (g * torch.sigmoid(g) * u).to(x_act.dtype).float()
                 y[lo:hi] = h @ down[e].float().t()
+        if defer_combine:
+            return y, inv
         return y[inv.long().view(T, k)].sum(1)
     assert x_act.is_contiguous() and gate.is_contiguous() and up.is_contiguous() and down.is_contiguous()
     assert gate.dtype == x_act.dtype and wts.dtype == torch.float32 and wts.is_contiguous()
@@ -306,5 +312,7 @@ def input_scaled_moe(x: torch.Tensor, x_act: torch.Tensor, ids: torch.Tensor, wt
     native.call("pkm_expert_gate_up", h.data_ptr(), x_act.data_ptr(), gate.data_ptr(), up.data_ptr(), offsets.data_ptr(),
                 sorted_.data_ptr(), wts.data_ptr(), n, k, E, F_, W, dt, st)
     native.call("pkm_expert_down", y.data_ptr(), h.data_ptr(), down.data_ptr(), offsets.data_ptr(), n, E, W, F_, dt, st)
+    if defer_combine:
+        return y, inv
     native.call("pkm_combine_rows", out.data_ptr(), y.data_ptr(), inv.data_ptr(), T, k, W, 1, st)
     return out

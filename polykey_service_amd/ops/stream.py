@@ -63,11 +63,15 @@ def save_last_rows(x: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, slo
 def sum_gain_norm(x: torch.Tensor, y: Optional[torch.Tensor], alpha: float, gain: torch.Tensor, eps: float,
                   out: Optional[torch.Tensor] = None, act_dtype: Optional[torch.dtype] = None,
                   rows: Optional[torch.Tensor] = None, hist: Optional[torch.Tensor] = None, nh: int = 0,
-                  coef: Optional[torch.Tensor] = None):
+                  coef: Optional[torch.Tensor] = None, gather: Optional[tuple] = None, save: Optional[tuple] = None):
     """z = (alpha x + y) / sqrt(mean((alpha x + y)^2) + eps) * gain (one number) in fp32.
 
     ``hist`` ([layers + 1, T_cap, W] fp32): z becomes entry ``nh - 1`` and the result is
     ``sum_j coef[j] hist[j]`` over the first ``nh`` entries.  ``rows``: only these rows of x.
+    ``gather`` = (inv [T * top] int32, top): y is a table of expert output rows and token t's y is
+    the plain sum of rows ``inv[t * top + j]`` (the MoE combine fused in; inv < 0: none).
+    ``save`` = (state, token_seq, cu_q, slots): the last token of every sequence in the step leaves
+    its x row in ``state[slots[s]]`` (the token-shift state, written after this step's shift read it).
     Returns (fp32 result written to ``out`` or None, copy in ``act_dtype`` or None)."""
     W = x.shape[1]
     R = rows.numel() if rows is not None else x.shape[0]
@@ -75,8 +79,14 @@ def sum_gain_norm(x: torch.Tensor, y: Optional[torch.Tensor], alpha: float, gain
     if not x.is_cuda:
         xs = x if rows is None else x[rows.long()]
         v = alpha * xs
-        if y is not None:
+        if gather is not None:
+            inv, top = gather
+            idx = inv.long().view(-1, top)
+            v = v + torch.where((idx >= 0)[..., None], y.float()[idx.clamp(min=0)], torch.zeros(())).sum(1)
+        elif y is not None:
             v = v + (y if rows is None else y[rows.long()]).float()
+        if save is not None:
+            save_last_rows(x, save[0], save[2], save[3], save[2].numel() - 1)
         z = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * gain
         if hist is not None:
             hist[nh - 1, :R] = z
@@ -87,12 +97,16 @@ def sum_gain_norm(x: torch.Tensor, y: Optional[torch.Tensor], alpha: float, gain
             act.copy_(z)
         return out, act
     assert x.dtype == torch.float32 and x.is_contiguous() and gain.dtype == torch.float32
-    assert y is None or (y.is_contiguous() and y.shape == x.shape)
+    assert y is None or (y.is_contiguous() and (gather is not None or y.shape == x.shape))
+    assert (gather is None and save is None) or rows is None
+    inv, top = gather if gather is not None else (None, 0)
+    state, token_seq, cu_q, slots = save if save is not None else (None, None, None, None)
     assert hist is None or (hist.dtype == torch.float32 and hist.is_contiguous() and rows is None and nh <= hist.shape[0]
                             and R <= hist.shape[1] and coef.dtype == torch.float32 and coef.numel() >= nh)
     dt = native.dt_code(act_dtype) if act_dtype is not None else 1
     native.call("pkm_sum_gain_norm", native.ptr(out), native.ptr(act), x.data_ptr(), native.ptr(y), native.ptr(rows),
                 float(alpha), gain.data_ptr(), float(eps), R, W, native.ptr(hist),
                 hist.stride(0) if hist is not None else 0, nh, native.ptr(coef), dt,
-                native.dt_code(y.dtype) if y is not None else -1, native.stream_ptr())
+                native.dt_code(y.dtype) if y is not None else -1, native.ptr(inv), top, native.ptr(state),
+                native.ptr(token_seq), native.ptr(cu_q), native.ptr(slots), native.stream_ptr())
     return out, act

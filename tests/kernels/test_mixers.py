@@ -225,3 +225,26 @@ def test_sigmoid_moe_on_grouped_mfma_gemms(E, k, F, W, T):
         err = (got.cpu() - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()
         assert float(err) < 1e-2, float(err)  # bf16 rounding of the scaled rows, h and y
         assert float((got.cpu() - want).abs().max()) < 0.05 * float(want.abs().max())
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_sum_gain_norm_fused_combine_and_state_save(dt):
+    dev = torch.device("cuda")
+    T, W, top = 9, 72, 2
+    x, yrows = torch.randn(T, W), torch.randn(T * top + 3, W).to(dt)
+    inv = torch.randperm(T * top + 3)[:T * top].to(torch.int32)
+    inv[5] = -1
+    g = torch.tensor([0.9])
+    m = batch_meta([4, 1, 4], [4, 20, 9], 4, torch.device("cpu"))
+    sl = torch.tensor([2, -1, 0], dtype=torch.int32)
+    st_c, st_g = torch.randn(3, W), None
+    st_g = st_c.to(dev)
+    w_out, w_act = stream.sum_gain_norm(x, yrows, 2.0, g, 1e-5, out=torch.zeros(T, W), act_dtype=dt, gather=(inv, top),
+                                        save=(st_c, m["tseq"], m["cu_q"], sl))
+    g_out, g_act = stream.sum_gain_norm(x.to(dev), yrows.to(dev), 2.0, g.to(dev), 1e-5, out=torch.zeros(T, W, device=dev),
+                                        act_dtype=dt, gather=(inv.to(dev), top),
+                                        save=(st_g, m["tseq"].to(dev), m["cu_q"].to(dev), sl.to(dev)))
+    torch.testing.assert_close(g_out.cpu(), w_out, rtol=2e-5, atol=2e-5)
+    torch.testing.assert_close(g_act.cpu().float(), w_act.float(), **tol(dt))
+    torch.testing.assert_close(st_g.cpu(), st_c)
+    assert torch.equal(st_c[2], x[3]) and torch.equal(st_c[0], x[8])
