@@ -240,16 +240,42 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
 
   for (int k0 = 0; k0 <= max_pos; k0 += BK) {
     const int nk = min(BK, max_pos + 1 - k0);
-    for (int c = tid; c < BK * R8; c += 256) {
-      const int key = c / R8, r8 = c - key * R8;
-      pk::u32x4 v = {0u, 0u, 0u, 0u};
-      if (key < nk) {
-        const int kp = k0 + key;
-        const int64_t slot = static_cast<int64_t>(bt[kp / block_size]) * block_size + kp % block_size;
-        v = *reinterpret_cast<const pk::u32x4*>(cache + slot * R + r8 * 8);
+    if (cache_t) {
+      // pages hold whole 32-key tiles: the tile is one contiguous run in each layout, and every
+      // thread's loads are issued before the first store (keys past the visible ones are stale
+      // cache rows: finite, and their weights are zero)
+      constexpr int NIT = (4 * R + 255) / 256;
+      const int64_t blk = bt[k0 / block_size];
+      const bf16_t* ksrc = cache + (blk * block_size + k0 % block_size) * R;
+      const bf16_t* tsrc = cache_t + (blk * (block_size / 32) + (k0 % block_size) / 32) * R * 32;
+      pk::u32x4 kv[NIT], tv[NIT];
+#pragma unroll
+      for (int i = 0; i < NIT; ++i) {
+        const int c = tid + 256 * i;
+        if (c < 4 * R) {
+          kv[i] = *reinterpret_cast<const pk::u32x4*>(ksrc + c * 8);
+          tv[i] = *reinterpret_cast<const pk::u32x4*>(tsrc + c * 8);
+        }
       }
-      *reinterpret_cast<pk::u32x4*>(cs + key * CS + r8 * 8) = v;
-      if (cache_t == nullptr) {  // no latent-major copy in the cache: transpose while staging
+#pragma unroll
+      for (int i = 0; i < NIT; ++i) {
+        const int c = tid + 256 * i;
+        if (c < 4 * R) {
+          const int key = c / R8, r8 = c - key * R8;
+          *reinterpret_cast<pk::u32x4*>(cs + key * CS + r8 * 8) = kv[i];
+          *reinterpret_cast<pk::u32x4*>(ct + (c >> 2) * CT + (c & 3) * 8) = tv[i];
+        }
+      }
+    } else {  // no latent-major copy in the cache: transpose while staging
+      for (int c = tid; c < BK * R8; c += 256) {
+        const int key = c / R8, r8 = c - key * R8;
+        pk::u32x4 v = {0u, 0u, 0u, 0u};
+        if (key < nk) {
+          const int kp = k0 + key;
+          const int64_t slot = static_cast<int64_t>(bt[kp / block_size]) * block_size + kp % block_size;
+          v = *reinterpret_cast<const pk::u32x4*>(cache + slot * R + r8 * 8);
+        }
+        *reinterpret_cast<pk::u32x4*>(cs + key * CS + r8 * 8) = v;
         bf16_t* dst = ct + (r8 * 8) * CT + key_slot(key);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -257,12 +283,6 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
           dst[(2 * e + 1) * CT] = static_cast<bf16_t>(v[e] >> 16);
         }
       }
-    }
-    if (cache_t) {  // the tile's latent-major copy is 64 contiguous bytes per latent coordinate
-      const bf16_t* src = cache_t + (static_cast<int64_t>(bt[k0 / block_size]) * (block_size / 32) +
-                                     (k0 % block_size) / 32) * R * 32;
-      for (int c = tid; c < R * 4; c += 256)
-        *reinterpret_cast<pk::u32x4*>(ct + (c >> 2) * CT + (c & 3) * 8) = *reinterpret_cast<const pk::u32x4*>(src + c * 8);
     }
     __syncthreads();
     if (__any(my_pos >= k0)) {
@@ -447,13 +467,21 @@ latent_merge_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t out_sh, co
   }
   __syncthreads();
   bf16_t* dst = out + static_cast<int64_t>(cu_q[s]) * out_st + static_cast<int64_t>(h) * out_sh;
-  for (int r = threadIdx.x; r < R; r += blockDim.x) {
-    float a = 0.f;
+  // four coordinates per thread; the runs' loads are independent of each other (an empty run's
+  // slab was never written: its value is discarded, not multiplied)
+  for (int r = 4 * threadIdx.x; r < R; r += 4 * blockDim.x) {
+    pk::f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
     for (int p = 0; p < n_parts; ++p) {
+      const pk::f32x4 v = *reinterpret_cast<const pk::f32x4*>(ws_o + (base + static_cast<int64_t>(p) * H) * R + r);
       const float w = wgt[p];
-      if (w != 0.f) a += w * ws_o[(base + static_cast<int64_t>(p) * H) * R + r];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) a[e] += w != 0.f ? w * v[e] : 0.f;
     }
-    dst[r] = pk::f2bf(a);
+    uint2 o2;
+    o2.x = pk::pack2(a[0], a[1]);
+    o2.y = pk::pack2(a[2], a[3]);
+    *reinterpret_cast<uint2*>(dst + r) = o2;
   }
 }
 

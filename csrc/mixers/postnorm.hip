@@ -79,7 +79,7 @@ struct NormFusion {
 };
 
 template <typename T, typename Y>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 sum_gain_norm_kernel(float* __restrict__ out, T* __restrict__ out_act, const float* __restrict__ x,
                      const Y* __restrict__ y, const int* __restrict__ rows, float alpha, const float* __restrict__ gain,
                      float eps, int W, float* __restrict__ hist, int64_t hist_stride, int nh,
@@ -169,8 +169,11 @@ PK_EXPORT int pkm_sum_gain_norm(void* out, void* out_act, const void* x, const v
   const NormFusion f{static_cast<const int*>(inv), top, static_cast<float*>(state), static_cast<const int*>(token_seq),
                      static_cast<const int*>(cu_q), static_cast<const int*>(slots)};
   const size_t lds = static_cast<size_t>(W) * sizeof(float);
+  // two coordinates per thread when the row allows: a token's chain of dependent loads (gathered
+  // expert rows, the history entries) is the latency of a decode-sized launch
+  const int threads = W >= 2048 ? 1024 : (W >= 1024 ? 512 : 256);
 #define PKM_SGN(E, Y)                                                                                             \
-  sum_gain_norm_kernel<E, Y><<<R, 256, lds, stream>>>(static_cast<float*>(out), static_cast<E*>(out_act),         \
+  sum_gain_norm_kernel<E, Y><<<R, threads, lds, stream>>>(static_cast<float*>(out), static_cast<E*>(out_act),         \
                                                       static_cast<const float*>(x), static_cast<const Y*>(y),     \
                                                       static_cast<const int*>(rows), alpha,                       \
                                                       static_cast<const float*>(gain), eps, W,                    \
