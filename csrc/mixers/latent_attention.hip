@@ -238,25 +238,30 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
   for (int rt = 0; rt < NRT; ++rt) o[rt] = pk::f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
 
+  // with the latent-major copy a tile is one contiguous run in each layout (pages hold whole 32-key
+  // tiles) and every thread's loads are issued before its first store; keys past the visible ones
+  // are stale cache rows: finite, and their weights are zero.  (Issuing tile t+1's loads before
+  // tile t's products costs 64 more live registers and the second workgroup per CU: measured slower.)
+  constexpr int NIT = (4 * R + 255) / 256;
+  pk::u32x4 kv[NIT], tv[NIT];
+  auto fetch = [&](int k0) {
+    const int64_t blk = bt[k0 / block_size];
+    const bf16_t* ksrc = cache + (blk * block_size + k0 % block_size) * R;
+    const bf16_t* tsrc = cache_t + (blk * (block_size / 32) + (k0 % block_size) / 32) * R * 32;
+#pragma unroll
+    for (int i = 0; i < NIT; ++i) {
+      const int c = tid + 256 * i;
+      if (c < 4 * R) {
+        kv[i] = *reinterpret_cast<const pk::u32x4*>(ksrc + c * 8);
+        tv[i] = *reinterpret_cast<const pk::u32x4*>(tsrc + c * 8);
+      }
+    }
+  };
+
   for (int k0 = 0; k0 <= max_pos; k0 += BK) {
     const int nk = min(BK, max_pos + 1 - k0);
     if (cache_t) {
-      // pages hold whole 32-key tiles: the tile is one contiguous run in each layout, and every
-      // thread's loads are issued before the first store (keys past the visible ones are stale
-      // cache rows: finite, and their weights are zero)
-      constexpr int NIT = (4 * R + 255) / 256;
-      const int64_t blk = bt[k0 / block_size];
-      const bf16_t* ksrc = cache + (blk * block_size + k0 % block_size) * R;
-      const bf16_t* tsrc = cache_t + (blk * (block_size / 32) + (k0 % block_size) / 32) * R * 32;
-      pk::u32x4 kv[NIT], tv[NIT];
-#pragma unroll
-      for (int i = 0; i < NIT; ++i) {
-        const int c = tid + 256 * i;
-        if (c < 4 * R) {
-          kv[i] = *reinterpret_cast<const pk::u32x4*>(ksrc + c * 8);
-          tv[i] = *reinterpret_cast<const pk::u32x4*>(tsrc + c * 8);
-        }
-      }
+      fetch(k0);
 #pragma unroll
       for (int i = 0; i < NIT; ++i) {
         const int c = tid + 256 * i;
@@ -287,12 +292,11 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
     __syncthreads();
     if (__any(my_pos >= k0)) {
       pk::f32x4 sa[2] = {pk::f32x4{0.f, 0.f, 0.f, 0.f}, pk::f32x4{0.f, 0.f, 0.f, 0.f}};
+      const bf16_t* kr = cs + n * CS + 8 * g;
 #pragma unroll
-      for (int sub = 0; sub < 2; ++sub) {
-        const bf16_t* kr = cs + (sub * 16 + n) * CS + 8 * g;
-#pragma unroll
-        for (int kk = 0; kk < NKK; ++kk)
-          sa[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(kr + kk * 32), qf[kk], sa[sub], 0, 0, 0);
+      for (int kk = 0; kk < NKK; ++kk) {  // the two 16-key halves alternate: two independent chains
+        sa[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(kr + kk * 32), qf[kk], sa[0], 0, 0, 0);
+        sa[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(kr + 16 * CS + kk * 32), qf[kk], sa[1], 0, 0, 0);
       }
       float sc[8];
       float tmax = -INFINITY;

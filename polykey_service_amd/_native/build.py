@@ -60,7 +60,8 @@ def targets() -> List[Target]:
         # mixers and residual-stream kernels built for bf16 and fp32 alike (latent attention, post-norm
         # stream, sigmoid-routed experts): a library of its own, so a model that needs only these
         # compiles only these on first use
-        Target("libpk_mixers", "hip", _g("csrc/mixers/*.hip"), _g("csrc/mixers/*.h") + [os.path.join(REPO, "csrc/kernels/common.h")]),
+        Target("libpk_mixers", "hip", _g("csrc/mixers/*.hip"), _g("csrc/mixers/*.h") + [os.path.join(REPO, "csrc/kernels/common.h")],
+               extra_flags=NO_PACKED_FP32),
         Target("libpk_comm", "hip", _g("csrc/comm/*.hip"), _g("csrc/comm/*.h")),
         Target("_pk_aesgcm", "pybind", _g("csrc/security/*.cpp"), _g("csrc/security/*.h"), ["crypto"]),
         Target("_pk_runtime", "pybind", _g("csrc/runtime/*.cpp"), _g("csrc/runtime/*.h")),
@@ -68,9 +69,10 @@ def targets() -> List[Target]:
 
 
 HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Wall", "-Wno-unused-function",
-             "-Wno-unused-variable", "-Wno-unused-result", "-ffp-contract=fast", "-munsafe-fp-atomics",
-             # the compiler forms no packed-fp32 instructions from scalar float code
-             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+             "-Wno-unused-variable", "-Wno-unused-result", "-ffp-contract=fast", "-munsafe-fp-atomics"]
+# the compiler forms no packed-fp32 instructions from scalar float code (libpk_mixers; the older
+# libraries keep the build their collectives and fused launches were validated with)
+NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-fvisibility=hidden"]
 if os.environ.get("POLYKEY_DEBUG_KERNELS", "0") == "1":  # device bounds asserts (PK_DEVICE_ASSERT)
     HIP_FLAGS = HIP_FLAGS + ["-DPK_DEBUG", "-g"]

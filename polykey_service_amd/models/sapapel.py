@@ -158,6 +158,8 @@ class SapapelForCausalLM(nn.Module):
         L.dwa = f32(get(p + "dwa")) if has(p + "dwa") else None
         if L.dwa is not None and L.dwa.numel() != i + 2:
             raise ValueError(f"{p}dwa has {L.dwa.numel()} entries, layer {i} averages {i + 2} outputs")
+        if L.mlp is None and has(p + "norm2"):  # a second norm without a feed-forward: it norms alpha x
+            L.g2 = f32(get(p + "norm2"))
         if L.mlp is not None:
             E = spec.mlp.experts
             L.g2 = f32(get(p + "norm2"))
@@ -294,6 +296,9 @@ class SapapelForCausalLM(nn.Module):
                                                       save=save)
                 y, inv = L.mlp(x1, x1_act, defer_combine=True)
                 x, _ = stream_ops.sum_gain_norm(x1, y, alpha, L.g2, eps, out=out, gather=(inv, L.mlp.spec.top), **depth)
+            elif L.g2 is not None:  # no feed-forward but a second norm: x <- norm2(alpha x1)
+                x1, _ = stream_ops.sum_gain_norm(x, m, alpha, L.g1, eps, out=torch.empty_like(x), save=save)
+                x, _ = stream_ops.sum_gain_norm(x1, None, alpha, L.g2, eps, out=out, **depth)
             else:
                 x, _ = stream_ops.sum_gain_norm(x, m, alpha, L.g1, eps, out=out, save=save, **depth)
             if L.dwa is None:  # later layers' averages still read this layer's output

@@ -285,13 +285,14 @@ def test_long_decoding_across_pages(device, small):
 @pytest.mark.parametrize("kw", [
     dict(width=40, heads=1, dim=16, vdim=4, kv_rank=33, ff=17, experts=3, top=1, alpha=1.0, layers=2),
     dict(width=64, heads=4, dim=4, vdim=4, kv_rank=8, ff=8, experts=4, top=4, alpha=0.5, layers=1, eps=1e-3),
-    dict(width=56, heads=2, dim=24, vdim=8, kv_rank=16, ff=30, experts=70, top=3, layers=4, mlp_none=(1,), scale=0.05),
+    dict(width=56, heads=2, dim=24, vdim=8, kv_rank=16, ff=30, experts=70, top=3, layers=4, mlp_none=(1, 3), scale=0.05),
 ])
 def test_other_sizes(device, tmp_path, kw):
     cfg = O.make_config(vocab=50, **kw)
     w = O.random_model(cfg, seed=7)
-    if kw.get("layers") == 4:  # a layer without shift and one without depth weights
-        del w["l2.shift"], w["l0.dwa"]
+    if kw.get("layers") == 4:  # a layer without shift, one without depth weights; of the two layers
+        del w["l2.shift"], w["l0.dwa"]  # without feed-forward, one still has its second norm
+        w["l3.norm2"] = torch.tensor(1.25)
     path = checkpoint(tmp_path, cfg, w)
     toks = rand_tokens(45, 50, 3)
     want = O.forward(toks, w, cfg)
@@ -331,3 +332,23 @@ def test_greedy_generation_through_the_scheduler(device, small):
     assert eng.bm.num_free == eng.bm.num_blocks and eng.bm.num_free_state_slots == 4
     if device == "cuda":
         assert eng.runner.stats["graph_steps"] > 0
+
+
+@pytest.mark.gpu
+def test_pipelined_decode_continuations(small):
+    """Overlapped engine steps: decode step k+1 is launched from step k's sampled ids while they are
+    still on the GPU (graph replays); the tokens equal the unpipelined engine's."""
+    cfg, w, path = small
+    prompts = [rand_tokens(n, cfg["vocab"], 60 + n) for n in (40, 7)]
+
+    def run(overlap):
+        ecfg = EngineConfig(model_path=path, dtype="float32", block_size=BS, max_num_seqs=4, max_num_batched_tokens=256,
+                            max_model_len=512, num_kv_blocks=16, watermark=0.0, hip_graphs=True, device="cuda",
+                            graph_batch_sizes=(1, 2, 4), overlap=overlap)
+        eng = LLMEngine(ecfg, ParallelState(device=torch.device("cuda")))
+        out = eng.generate(prompts, SamplingParams(max_tokens=24, ignore_eos=True))
+        return out, eng.continuation_steps
+
+    plain, _ = run(False)
+    piped, n_cont = run(True)
+    assert piped == plain and n_cont > 0

@@ -78,6 +78,8 @@ def layer(x: torch.Tensor, w: Dict[str, torch.Tensor], i: int, cfg: dict) -> tor
     x = gain_rms_norm(alpha * x + latent_attention(h, w, p + "mix.", lc["mixer"], eps), w[p + "norm1"], eps)
     if lc.get("mlp") is not None:
         x = gain_rms_norm(alpha * x + feed_forward(x, w, p + "mlp.", lc["mlp"]), w[p + "norm2"], eps)
+    elif p + "norm2" in w:  # no feed-forward: the second sum is alpha x alone
+        x = gain_rms_norm(alpha * x, w[p + "norm2"], eps)
     return x
 
 
