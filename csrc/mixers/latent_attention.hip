@@ -184,7 +184,8 @@ latent_attention_kernel(T* __restrict__ out, int64_t out_st, int64_t out_sh, con
 }
 
 // ---- bf16 on the matrix cores -------------------------------------------------------------------
-// 64 (token, head) rows per workgroup, 16 per wave; 32-key tiles.  Both products run transposed on
+// 128 (token, head) rows per workgroup, 16 per wave; 32-key tiles (the cached tile is re-read by
+// every workgroup of a sequence, so rows per workgroup set the kernel's memory traffic).  Both products run transposed on
 // mfma_f32_16x16x32_bf16 so that the softmax weights never leave their registers:
 //
 //   S^T [keys x rows] = C [keys x R] . Q~^T     A = key rows from LDS `cs`, B = the wave's Q~ (registers)
@@ -195,14 +196,17 @@ latent_attention_kernel(T* __restrict__ out, int64_t out_st, int64_t out_sh, con
 // of the second product wants 8 key slots per lane, so slot (g, e) is key 4g+e of the first half
 // for e < 4 and key 16+4g+e-4 of the second, and `ct` stores its columns in that slot order.
 // The tile is staged twice (key-major and latent-major) because it is both the key and the value.
+// threads of the prompt kernel: 8 waves = 128 (token, head) rows per workgroup share every staged tile
+constexpr int kPromptThreads = 512;
+
 template <int R>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kPromptThreads)
 latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t out_sh, const bf16_t* __restrict__ q,
                              int64_t q_st, int64_t q_sh, const bf16_t* __restrict__ cache,
                              const bf16_t* __restrict__ cache_t, const int* __restrict__ block_tables, int max_blocks,
                              const int* __restrict__ cu_q, const int* __restrict__ context_lens, int n_seqs, int H,
                              int block_size, float scale) {
-  constexpr int BQ = 64, BK = 32, NKK = R / 32, NRT = R / 16, CS = R + 8, CT = BK + 8, R8 = R / 8;
+  constexpr int NT = kPromptThreads, BQ = NT / 4, BK = 32, NKK = R / 32, NRT = R / 16, CS = R + 8, CT = BK + 8, R8 = R / 8;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t* cs = reinterpret_cast<bf16_t*>(smem_raw);  // [BK][CS]   key-major
   bf16_t* ct = cs + BK * CS;                          // [R][CT]    latent-major, key slots permuted
@@ -240,9 +244,10 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
 
   // with the latent-major copy a tile is one contiguous run in each layout (pages hold whole 32-key
   // tiles) and every thread's loads are issued before its first store; keys past the visible ones
-  // are stale cache rows: finite, and their weights are zero.  (Issuing tile t+1's loads before
-  // tile t's products costs 64 more live registers and the second workgroup per CU: measured slower.)
-  constexpr int NIT = (4 * R + 255) / 256;
+  // are stale cache rows: finite, and their weights are zero.  Issuing tile t+1's loads before tile
+  // t's products was tried twice: at 4 waves it cost the second workgroup per CU (slower), at 8
+  // waves and a 512-wide latent the extra live registers spill (the compiler's resource report).
+  constexpr int NIT = (4 * R + NT - 1) / NT;
   pk::u32x4 kv[NIT], tv[NIT];
   auto fetch = [&](int k0) {
     const int64_t blk = bt[k0 / block_size];
@@ -250,7 +255,7 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
     const bf16_t* tsrc = cache_t + (blk * (block_size / 32) + (k0 % block_size) / 32) * R * 32;
 #pragma unroll
     for (int i = 0; i < NIT; ++i) {
-      const int c = tid + 256 * i;
+      const int c = tid + NT * i;
       if (c < 4 * R) {
         kv[i] = *reinterpret_cast<const pk::u32x4*>(ksrc + c * 8);
         tv[i] = *reinterpret_cast<const pk::u32x4*>(tsrc + c * 8);
@@ -264,7 +269,7 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
       fetch(k0);
 #pragma unroll
       for (int i = 0; i < NIT; ++i) {
-        const int c = tid + 256 * i;
+        const int c = tid + NT * i;
         if (c < 4 * R) {
           const int key = c / R8, r8 = c - key * R8;
           *reinterpret_cast<pk::u32x4*>(cs + key * CS + r8 * 8) = kv[i];
@@ -272,7 +277,7 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
         }
       }
     } else {  // no latent-major copy in the cache: transpose while staging
-      for (int c = tid; c < BK * R8; c += 256) {
+      for (int c = tid; c < BK * R8; c += NT) {
         const int key = c / R8, r8 = c - key * R8;
         pk::u32x4 v = {0u, 0u, 0u, 0u};
         if (key < nk) {
@@ -292,11 +297,12 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
     __syncthreads();
     if (__any(my_pos >= k0)) {
       pk::f32x4 sa[2] = {pk::f32x4{0.f, 0.f, 0.f, 0.f}, pk::f32x4{0.f, 0.f, 0.f, 0.f}};
-      const bf16_t* kr = cs + n * CS + 8 * g;
 #pragma unroll
-      for (int kk = 0; kk < NKK; ++kk) {  // the two 16-key halves alternate: two independent chains
-        sa[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(kr + kk * 32), qf[kk], sa[0], 0, 0, 0);
-        sa[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(kr + 16 * CS + kk * 32), qf[kk], sa[1], 0, 0, 0);
+      for (int sub = 0; sub < 2; ++sub) {
+        const bf16_t* kr = cs + (sub * 16 + n) * CS + 8 * g;
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk)
+          sa[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(kr + kk * 32), qf[kk], sa[sub], 0, 0, 0);
       }
       float sc[8];
       float tmax = -INFINITY;
@@ -519,8 +525,9 @@ static int launch_latent_mfma(void* out, long long out_st, long long out_sh, con
                                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     if (e != hipSuccess) return static_cast<int>(e);
   }
-  const int grid = static_cast<int>((static_cast<int64_t>(T) * H + 63) / 64 + n_seqs);
-  kern<<<grid, 256, lds, stream>>>(static_cast<bf16_t*>(out), out_st, out_sh, static_cast<const bf16_t*>(q), q_st, q_sh,
+  constexpr int BQ = kPromptThreads / 4;
+  const int grid = static_cast<int>((static_cast<int64_t>(T) * H + BQ - 1) / BQ + n_seqs);
+  kern<<<grid, kPromptThreads, lds, stream>>>(static_cast<bf16_t*>(out), out_st, out_sh, static_cast<const bf16_t*>(q), q_st, q_sh,
                                    static_cast<const bf16_t*>(cache), static_cast<const bf16_t*>(cache_t),
                                    static_cast<const int*>(block_tables), max_blocks, static_cast<const int*>(cu_q),
                                    static_cast<const int*>(context_lens), n_seqs, H, block_size, scale);

@@ -69,7 +69,11 @@ __global__ void __launch_bounds__(256) save_last_rows_kernel(float* __restrict__
 //   state (token_seq, cu_q, slots): a token that is the last of its sequence in this step leaves its
 //                       x row in the sequence's state slot (the token shift of the NEXT step reads it;
 //                       this step's shift has already run)
+//   slabs (nslab, slab_stride): y is nslab split-K slabs [nslab][rows][W] of a projection and the
+//                       token's y is their sum (the slab reduce of the decode GEMM fused in)
 struct NormFusion {
+  int nslab;
+  int64_t slab_stride;
   const int* inv;
   int top;
   float* state;
@@ -99,6 +103,7 @@ sum_gain_norm_kernel(float* __restrict__ out, T* __restrict__ out_act, const flo
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
     const float xv = xr[i];
     float yv = yr ? ld<Y>(yr + i) : 0.f;
+    for (int sl = 1; sl < f.nslab; ++sl) yv += ld<Y>(yr + sl * f.slab_stride + i);
     if (f.inv) {
       for (int j = 0; j < f.top; ++j) {
         const int yrow = f.inv[src * f.top + j];
@@ -160,13 +165,13 @@ PK_EXPORT int pkm_save_last_rows(void* state, const void* x, const void* cu_q, c
 // gathered (see NormFusion); state != nullptr: last rows are saved (token_seq, cu_q, slots given).
 PK_EXPORT int pkm_sum_gain_norm(void* out, void* out_act, const void* x, const void* y, const void* rows, float alpha,
                                 const void* gain, float eps, int R, int W, void* hist, long long hist_stride, int nh,
-                                const void* coef, int dt, int y_dt, const void* inv, int top, void* state,
+                                const void* coef, int dt, int y_dt, int nslab, const void* inv, int top, void* state,
                                 const void* token_seq, const void* cu_q, const void* slots, hipStream_t stream) {
   if (R <= 0) return 0;
   if (hist && (nh < 1 || !coef)) return -1;
   if ((inv && (!y || top < 1 || rows)) || (state && (!token_seq || !cu_q || !slots || rows))) return -1;
-  if (W > 16384) return -1;
-  const NormFusion f{static_cast<const int*>(inv), top, static_cast<float*>(state), static_cast<const int*>(token_seq),
+  if (W > 16384 || nslab < 1 || (nslab > 1 && (!y || inv || rows))) return -1;
+  const NormFusion f{nslab, static_cast<int64_t>(R) * W, static_cast<const int*>(inv), top, static_cast<float*>(state), static_cast<const int*>(token_seq),
                      static_cast<const int*>(cu_q), static_cast<const int*>(slots)};
   const size_t lds = static_cast<size_t>(W) * sizeof(float);
   // two coordinates per thread when the row allows: a token's chain of dependent loads (gathered

@@ -57,6 +57,7 @@ class LatentAttention(nn.Module):
         self.uk = None        # [H, D, R]
         self.uv_t = None      # [H, R, V]
         self.w_o = None       # [W, H*V]
+        self.w_in_p = self.w_o_p = None  # block-packed copies for the decode GEMM (pack())
 
     def set(self, q, dkv, latent_w, uk, uv, g, o, dtype, device) -> None:
         s = self.spec
@@ -70,18 +71,43 @@ class LatentAttention(nn.Module):
         self.uv_t = _p(to(uv).view(H, V, R).transpose(1, 2))
         self.w_o = _p(to(o))
 
+    def pack(self) -> None:
+        """Block-packed copies of the two projections where the decode GEMM tiles them."""
+        ok = lambda w: w.is_cuda and w.dtype == torch.bfloat16 and w.shape[0] % 128 == 0 and w.shape[1] % 256 == 0
+        if self.w_in_p is None and ok(self.w_in):
+            self.w_in_p = gemm.pack_weight(self.w_in)
+        if self.w_o_p is None and ok(self.w_o):
+            self.w_o_p = gemm.pack_weight(self.w_o)
+
+    @staticmethod
+    def _split_k(x: torch.Tensor, w: torch.Tensor, packed: Optional[torch.Tensor]):
+        """Decode-sized rows on shapes the weight-streaming GEMM tiles: its split-K slabs, unreduced
+        (gemm.Partial), so the launch fills the chip; None otherwise."""
+        if not gemm.skinny_ok(x, w):
+            return None
+        S = gemm.choose_split(w.shape[0], x.shape[1], x.shape[0])
+        if S <= 1:
+            return None
+        ws = torch.empty(S * x.shape[0] * w.shape[0], dtype=torch.float32, device=x.device)
+        return gemm.linear_partial(x, w, ws, S, packed=packed)
+
     def forward(self, h: torch.Tensor, md, cache: torch.Tensor, eps: float,
-                cache_t: Optional[torch.Tensor] = None) -> torch.Tensor:
+                cache_t: Optional[torch.Tensor] = None):
+        """The mixer's output [T, W], or for decode-sized steps the output projection's unreduced
+        split-K slabs (gemm.Partial) for the norm kernel that follows to sum."""
         s = self.spec
         H, D, V, R = s.heads, s.dim, s.vdim, s.kv_rank
         T = h.shape[0]
-        qdg = gemm.linear(h, self.w_in)
+        part = self._split_k(h, self.w_in, self.w_in_p)
+        qdg = gemm.reduce_partial(part) if part is not None else gemm.linear(h, self.w_in, packed=self.w_in_p)
         la_ops.latent_norm_cache(qdg[:, H * D:H * D + R], self.latent_w, eps, cache, md.slot_mapping, cache_t)
         q_lat = torch.bmm(qdg[:, :H * D].view(T, H, D).transpose(0, 1), self.uk)          # [H, T, R]
         o_lat = la_ops.latent_attention(q_lat, cache, md.block_tables, md.cu_q, md.context_lens, md.num_seqs, s.scale,
                                         cache_t, md.num_decode)
         o = torch.bmm(o_lat, self.uv_t)                                                    # [H, T, V]
-        return gemm.linear(la_ops.gate_merge(o, qdg[:, H * D + R:]), self.w_o)
+        a = la_ops.gate_merge(o, qdg[:, H * D + R:])
+        part = self._split_k(a, self.w_o, self.w_o_p)
+        return part if part is not None else gemm.linear(a, self.w_o, packed=self.w_o_p)
 
 
 class SigmoidMoE(nn.Module):
@@ -226,6 +252,7 @@ class SapapelForCausalLM(nn.Module):
     def pack_decode_weights(self) -> None:
         """Block-packed copies of the expert weights for the decode GEMM (engine hook)."""
         for L in self.layers:
+            L.mix.pack()
             if L.mlp is not None:
                 L.mlp.pack()
 

@@ -72,7 +72,7 @@ MIXER_SIGNATURES = {
     "pkm_embed_rows": [P, P, P, I32, I32, I32, I32, P],
     "pkm_token_shift": [P, P, P, P, P, P, P, P, I32, I32, I32, P],
     "pkm_save_last_rows": [P, P, P, P, I32, I32, P],
-    "pkm_sum_gain_norm": [P, P, P, P, P, F32, P, F32, I32, I32, P, I64, I32, P, I32, I32, P, I32, P, P, P, P, P],
+    "pkm_sum_gain_norm": [P, P, P, P, P, F32, P, F32, I32, I32, P, I64, I32, P, I32, I32, I32, P, I32, P, P, P, P, P],
     "pkm_latent_norm_cache": [P, P, I32, P, I64, P, P, I32, I32, F32, I32, P],
     "pkm_latent_attention": [P, I64, I64, P, I64, I64, P, P, P, I32, P, P, I32, I32, I32, I32, I32, F32, I32, P],
     "pkm_latent_decode": [P, I64, I64, P, I64, I64, P, P, P, I32, P, P, I32, I32, I32, I32, F32, P, P, I32, I32, P],

@@ -11,7 +11,7 @@ from typing import Optional
 
 import torch
 
-from . import native
+from . import gemm, native
 
 
 def embed_rows(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -72,8 +72,13 @@ def sum_gain_norm(x: torch.Tensor, y: Optional[torch.Tensor], alpha: float, gain
     the plain sum of rows ``inv[t * top + j]`` (the MoE combine fused in; inv < 0: none).
     ``save`` = (state, token_seq, cu_q, slots): the last token of every sequence in the step leaves
     its x row in ``state[slots[s]]`` (the token-shift state, written after this step's shift read it).
+    ``y`` may also be the decode GEMM's unreduced split-K slabs (``gemm.Partial``): their sum is y.
     Returns (fp32 result written to ``out`` or None, copy in ``act_dtype`` or None)."""
     W = x.shape[1]
+    nslab = 1
+    if isinstance(y, gemm.Partial):
+        assert x.is_cuda and y.M == x.shape[0] and y.N == W and gather is None and rows is None
+        nslab, y = y.S, y.view()[0]  # the first slab; the others follow at M * W elements each
     R = rows.numel() if rows is not None else x.shape[0]
     act = torch.empty((R, W), dtype=act_dtype, device=x.device) if act_dtype is not None else None
     if not x.is_cuda:
@@ -97,7 +102,7 @@ def sum_gain_norm(x: torch.Tensor, y: Optional[torch.Tensor], alpha: float, gain
             act.copy_(z)
         return out, act
     assert x.dtype == torch.float32 and x.is_contiguous() and gain.dtype == torch.float32
-    assert y is None or (y.is_contiguous() and (gather is not None or y.shape == x.shape))
+    assert y is None or (y.is_contiguous() and (gather is not None or nslab > 1 or y.shape == x.shape))
     assert (gather is None and save is None) or rows is None
     inv, top = gather if gather is not None else (None, 0)
     state, token_seq, cu_q, slots = save if save is not None else (None, None, None, None)
@@ -107,6 +112,6 @@ def sum_gain_norm(x: torch.Tensor, y: Optional[torch.Tensor], alpha: float, gain
     native.call("pkm_sum_gain_norm", native.ptr(out), native.ptr(act), x.data_ptr(), native.ptr(y), native.ptr(rows),
                 float(alpha), gain.data_ptr(), float(eps), R, W, native.ptr(hist),
                 hist.stride(0) if hist is not None else 0, nh, native.ptr(coef), dt,
-                native.dt_code(y.dtype) if y is not None else -1, native.ptr(inv), top, native.ptr(state),
+                native.dt_code(y.dtype) if y is not None else -1, nslab, native.ptr(inv), top, native.ptr(state),
                 native.ptr(token_seq), native.ptr(cu_q), native.ptr(slots), native.stream_ptr())
     return out, act

@@ -352,3 +352,28 @@ def test_pipelined_decode_continuations(small):
     plain, _ = run(False)
     piped, n_cont = run(True)
     assert piped == plain and n_cont > 0
+
+
+@pytest.mark.gpu
+def test_aligned_sizes_on_the_matrix_core_paths(tmp_path):
+    """Sizes that every fast path tiles (bf16): MFMA latent attention for prompts and decoding with
+    the latent-major cache copy, grouped MFMA expert GEMMs on scaled rows, split-K decode
+    projections summed inside the norm kernel.  Against the fp32 model within bf16 rounding, for a
+    prompt in portions, decoded tokens, and a second request sharing the steps."""
+    cfg = O.make_config(vocab=128, width=256, layers=2, heads=2, dim=64, vdim=128, kv_rank=128, ff=256, experts=4, top=2)
+    w = O.random_model(cfg, seed=11, std=0.04)
+    path = checkpoint(tmp_path, cfg, w)
+    eng = engine(path, "cuda", dtype="bfloat16", graphs=True)
+    L = eng.model.layers[0]
+    assert L.mlp.w13 is not None and L.mlp.w13_p is not None and L.mix.w_o_p is not None
+    assert eng.runner.kv_caches[0][1] is not None  # the latent-major copy
+    a, b = rand_tokens(150, 128, 1), rand_tokens(40, 128, 2)
+    want = {"a": O.forward(a, w, cfg), "b": O.forward(b, w, cfg)}
+    pa, pb = cut("a", a, [70, 2, 50]), cut("b", b, [33])
+    steps = [[pa.pop(0)]] + [[x, y] for x, y in zip(pa, pb)] + [[x] for x in pa[len(pb):]]
+    got = replay(eng, steps)
+    assert eng.runner.stats["graph_steps"] > 0
+    for k, toks in (("a", a), ("b", b)):
+        err = torch.stack([got[k][p] - want[k][p] for p in range(len(toks))])
+        assert float(err.pow(2).mean().sqrt()) < 0.04 * float(want[k].pow(2).mean().sqrt())
+        assert float(err.abs().max()) < 0.25 * float(want[k].abs().max())
