@@ -363,7 +363,9 @@ def test_aligned_sizes_on_the_matrix_core_paths(tmp_path):
     cfg = O.make_config(vocab=128, width=256, layers=2, heads=2, dim=64, vdim=128, kv_rank=128, ff=256, experts=4, top=2)
     w = O.random_model(cfg, seed=11, std=0.04)
     path = checkpoint(tmp_path, cfg, w)
-    eng = engine(path, "cuda", dtype="bfloat16", graphs=True)
+    eng = engine(path, "cuda", dtype="bfloat16")
+    eng.runner.cfg.hip_graphs = True  # decode graphs whose logits stay readable, as bin/trace_run captures them
+    eng.runner.capture_graphs([1, 2, 4], keep_logits=True)
     L = eng.model.layers[0]
     assert L.mlp.w13 is not None and L.mlp.w13_p is not None and L.mix.w_o_p is not None
     assert eng.runner.kv_caches[0][1] is not None  # the latent-major copy
