@@ -183,6 +183,14 @@ latent_attention_kernel(T* __restrict__ out, int64_t out_st, int64_t out_sh, con
   }
 }
 
+// Softmax bookkeeping of the matrix-core kernels.  Scores are kept in log2 units (scale * log2 e
+// folded into one multiply).  The running reference m only moves when a tile's maximum exceeds it
+// by more than kLazyMax: weights are then at most 2^kLazyMax (exact in fp32, and in bf16 as the
+// second product's operand), the softmax is unchanged (any reference gives the same quotient),
+// and the 128-register rescale of the output tile runs on a few tiles instead of nearly all.
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLazyMax = 10.f;
+
 // ---- bf16 on the matrix cores -------------------------------------------------------------------
 // 128 (token, head) rows per workgroup, 16 per wave; 32-key tiles (the cached tile is re-read by
 // every workgroup of a sequence, so rows per workgroup set the kernel's memory traffic).  Both products run transposed on
@@ -241,6 +249,7 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
 #pragma unroll
   for (int rt = 0; rt < NRT; ++rt) o[rt] = pk::f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
+  const float scale2 = scale * kLog2e;  // scores in log2 units: a weight is one exp2
 
   // with the latent-major copy a tile is one contiguous run in each layout (pages hold whole 32-key
   // tiles) and every thread's loads are issued before its first store; keys past the visible ones
@@ -309,21 +318,21 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int key = k0 + (e >> 2) * 16 + 4 * g + (e & 3);
-        sc[e] = key <= my_pos ? sa[e >> 2][e & 3] * scale : -INFINITY;
+        sc[e] = key <= my_pos ? sa[e >> 2][e & 3] * scale2 : -INFINITY;
         tmax = fmaxf(tmax, sc[e]);
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m_run, tmax);
+      const float m_new = tmax > m_run + kLazyMax ? tmax : m_run;  // the reference moves only on a real jump
       float p[8], tsum = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        p[e] = sc[e] == -INFINITY ? 0.f : expf(sc[e] - m_new);
+        p[e] = sc[e] == -INFINITY ? 0.f : exp2f(sc[e] - m_new);
         tsum += p[e];
       }
       tsum += __shfl_xor(tsum, 16, 64);
       tsum += __shfl_xor(tsum, 32, 64);
-      const float resc = m_run == -INFINITY ? (m_new == -INFINITY ? 1.f : 0.f) : expf(m_run - m_new);
+      const float resc = m_run == -INFINITY ? (m_new == -INFINITY ? 1.f : 0.f) : exp2f(m_run - m_new);
       m_run = m_new;
       l_run = l_run * resc + tsum;
       pk::u32x4 pw;
@@ -352,6 +361,172 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
       *reinterpret_cast<uint2*>(dst + rt * 16) = w;
     }
   }
+}
+
+// ---- the 512-wide latent: tiles staged by LDS-DMA into two buffers ------------------------------
+// At R = 512 a wave's 16 rows hold 128 output accumulators and 64 registers of folded queries, so
+// there is no room to keep the next tile in registers and only two waves fit a SIMD: the tile loads
+// go straight to LDS instead (buffer_load ... lds, no VGPRs), tile t+1 into the other buffer while
+// tile t's products run, one barrier per tile.  A wave instruction moves 1 KiB: exactly one
+// key-major row (padded to 1040 B in LDS through the instruction's LDS base), or 16 rows of the
+// latent-major copy, whose 16-byte parts are XOR-swizzled by the row on the GLOBAL side of the
+// copy (lane l fetches part (l & 3) ^ ((l >> 3) & 3) of row l >> 2) so that the unpadded 64-byte
+// rows read conflict-free.  Needs the latent-major cache copy (pages of whole 32-key tiles).
+__global__ void __launch_bounds__(kPromptThreads)
+latent_attention_dma512_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t out_sh, const bf16_t* __restrict__ q,
+                               int64_t q_st, int64_t q_sh, const bf16_t* __restrict__ cache,
+                               const bf16_t* __restrict__ cache_t, const int* __restrict__ block_tables, int max_blocks,
+                               const int* __restrict__ cu_q, const int* __restrict__ context_lens, int n_seqs, int H,
+                               int block_size, float scale) {
+  constexpr int R = 512, NT = kPromptThreads, BQ = NT / 4, BK = 32, NKK = R / 32, NRT = R / 16, CS = R + 8;
+  constexpr int kCsBytes = BK * CS * 2, kCtBytes = R * BK * 2, kBuf = kCsBytes + kCtBytes;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  int s = 0, tile = blockIdx.x;
+  for (; s < n_seqs; ++s) {
+    const int nt = ((cu_q[s + 1] - cu_q[s]) * H + BQ - 1) / BQ;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (s >= n_seqs) return;
+  const int q0 = cu_q[s], qlen = cu_q[s + 1] - q0, ctx = context_lens[s];
+  const int n_rows = qlen * H, row0 = tile * BQ;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, n = lane & 15;
+  const int wu = __builtin_amdgcn_readfirstlane(wave);
+  const int* bt = block_tables + static_cast<int64_t>(s) * max_blocks;
+  const int my_row = row0 + 16 * wave + n;
+  const bool valid = my_row < n_rows;
+  const int tl = valid ? my_row / H : 0, h = valid ? my_row - tl * H : 0;
+  const int my_pos = valid ? ctx - qlen + tl : -1;
+  const int max_pos = ctx - qlen + (min(row0 + BQ, n_rows) - 1) / H;
+
+  pk::bf16x8_t qf[NKK];
+  {
+    const bf16_t* qr = q + static_cast<int64_t>(q0 + tl) * q_st + static_cast<int64_t>(h) * q_sh + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      pk::u32x4 v = {0u, 0u, 0u, 0u};
+      if (valid) v = *reinterpret_cast<const pk::u32x4*>(qr + kk * 32);
+      qf[kk] = __builtin_bit_cast(pk::bf16x8_t, v);
+    }
+  }
+  pk::f32x4 o[NRT];
+#pragma unroll
+  for (int rt = 0; rt < NRT; ++rt) o[rt] = pk::f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  const float scale2 = scale * kLog2e;  // scores in log2 units: a weight is one exp2
+
+  // lane offsets of the two copies: key-major rows are taken as they lie, latent-major parts swizzled
+  const unsigned kvo = static_cast<unsigned>(lane) * 16u;
+  const unsigned tvo = static_cast<unsigned>(((lane >> 2) * 4 + ((lane & 3) ^ ((lane >> 3) & 3))) * 16);
+  auto issue = [&](int k0, int buf) {  // this wave's 4 + 4 KiB of the tile at k0
+    const int blk = __builtin_amdgcn_readfirstlane(bt[k0 / block_size]);
+    const int kin = k0 % block_size;
+    const bf16_t* ksrc = cache + (static_cast<int64_t>(blk) * block_size + kin) * R;
+    const bf16_t* tsrc = cache_t + (static_cast<int64_t>(blk) * (block_size / 32) + kin / 32) * R * 32;
+    const auto krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(ksrc), static_cast<short>(0), kCtBytes, 0x00020000);
+    const auto trs = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(tsrc), static_cast<short>(0), kCtBytes, 0x00020000);
+    unsigned char* base = smem_raw + buf * kBuf;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = wu * 4 + j;  // key row / 16-row block of the latent-major copy
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(krs, (__attribute__((address_space(3))) void*)(base + row * (CS * 2)), 16, kvo,
+                                               static_cast<unsigned>(row) * 1024u, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(trs, (__attribute__((address_space(3))) void*)(base + kCsBytes + row * 1024),
+                                               16, tvo, static_cast<unsigned>(row) * 1024u, 0, 0);
+    }
+  };
+  if (max_pos >= 0) issue(0, 0);
+  int buf = 0;
+  for (int k0 = 0; k0 <= max_pos; k0 += BK, buf ^= 1) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // tile k0 has landed for every wave, and nobody still reads the other buffer
+    if (k0 + BK <= max_pos) issue(k0 + BK, buf ^ 1);
+    if (__any(my_pos >= k0)) {
+      const bf16_t* cs = reinterpret_cast<const bf16_t*>(smem_raw + buf * kBuf);
+      const bf16_t* ct = reinterpret_cast<const bf16_t*>(smem_raw + buf * kBuf + kCsBytes);
+      pk::f32x4 sa[2] = {pk::f32x4{0.f, 0.f, 0.f, 0.f}, pk::f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        const bf16_t* kr = cs + (sub * 16 + n) * CS + 8 * g;
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk)
+          sa[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(kr + kk * 32), qf[kk], sa[sub], 0, 0, 0);
+      }
+      float sc[8];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = k0 + (e >> 2) * 16 + 4 * g + (e & 3);
+        sc[e] = key <= my_pos ? sa[e >> 2][e & 3] * scale2 : -INFINITY;
+        tmax = fmaxf(tmax, sc[e]);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = tmax > m_run + kLazyMax ? tmax : m_run;  // the reference moves only on a real jump
+      float p[8], tsum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p[e] = sc[e] == -INFINITY ? 0.f : exp2f(sc[e] - m_new);
+        tsum += p[e];
+      }
+      tsum += __shfl_xor(tsum, 16, 64);
+      tsum += __shfl_xor(tsum, 32, 64);
+      const float resc = m_run == -INFINITY ? (m_new == -INFINITY ? 1.f : 0.f) : exp2f(m_run - m_new);
+      m_run = m_new;
+      l_run = l_run * resc + tsum;
+      pk::u32x4 pw;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pw[e] = pk::pack2(p[2 * e], p[2 * e + 1]);
+      const pk::bf16x8_t pb = __builtin_bit_cast(pk::bf16x8_t, pw);
+      if (__any(resc != 1.f)) {
+#pragma unroll
+        for (int rt = 0; rt < NRT; ++rt) o[rt] *= resc;
+      }
+      // row rt*16 + n of the latent-major tile, part g, at its swizzled place
+      const bf16_t* vr = ct + (n * 4 + (g ^ ((n >> 1) & 3))) * 8;
+#pragma unroll
+      for (int rt = 0; rt < NRT; ++rt)
+        o[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(vr + rt * 16 * 32), pb, o[rt], 0, 0, 0);
+    }
+  }
+  if (valid) {
+    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    bf16_t* dst = out + static_cast<int64_t>(q0 + tl) * out_st + static_cast<int64_t>(h) * out_sh + 4 * g;
+#pragma unroll
+    for (int rt = 0; rt < NRT; ++rt) {
+      uint2 w;
+      w.x = pk::pack2(o[rt][0] * inv, o[rt][1] * inv);
+      w.y = pk::pack2(o[rt][2] * inv, o[rt][3] * inv);
+      *reinterpret_cast<uint2*>(dst + rt * 16) = w;
+    }
+  }
+}
+
+static int g_latent_dma = 1;  // 0: the 512-wide latent takes the register-staged kernel too (tests)
+PK_EXPORT int pkm_set_latent_dma(int on) {
+  g_latent_dma = on;
+  return 0;
+}
+
+static int launch_latent_dma512(void* out, long long out_st, long long out_sh, const void* q, long long q_st,
+                                long long q_sh, const void* cache, const void* cache_t, const void* block_tables,
+                                int max_blocks, const void* cu_q, const void* context_lens, int n_seqs, int T, int H,
+                                int block_size, float scale, hipStream_t stream) {
+  constexpr int lds = 2 * (32 * 520 * 2 + 512 * 32 * 2);
+  static bool attr_set = false;
+  if (!attr_set) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(latent_attention_dma512_kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return static_cast<int>(e);
+    attr_set = true;
+  }
+  constexpr int BQ = kPromptThreads / 4;
+  const int grid = static_cast<int>((static_cast<int64_t>(T) * H + BQ - 1) / BQ + n_seqs);
+  latent_attention_dma512_kernel<<<grid, kPromptThreads, lds, stream>>>(
+      static_cast<bf16_t*>(out), out_st, out_sh, static_cast<const bf16_t*>(q), q_st, q_sh,
+      static_cast<const bf16_t*>(cache), static_cast<const bf16_t*>(cache_t), static_cast<const int*>(block_tables),
+      max_blocks, static_cast<const int*>(cu_q), static_cast<const int*>(context_lens), n_seqs, H, block_size, scale);
+  return PK_CHECK_LAUNCH();
 }
 
 // ---- decoding on the matrix cores -----------------------------------------------------------------
@@ -400,6 +575,7 @@ latent_decode_mfma_kernel(float* __restrict__ ws_o, float* __restrict__ ws_ml, c
 #pragma unroll
     for (int rt = 0; rt < NRT; ++rt) o[rt] = pk::f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
+  const float scale2 = scale * kLog2e;  // scores in log2 units: a weight is one exp2
     for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
       pk::f32x4 sa[2] = {pk::f32x4{0.f, 0.f, 0.f, 0.f}, pk::f32x4{0.f, 0.f, 0.f, 0.f}};
       const int blk = bt[k0 / block_size];
@@ -415,21 +591,21 @@ latent_decode_mfma_kernel(float* __restrict__ ws_o, float* __restrict__ ws_ml, c
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int key = k0 + (e >> 2) * 16 + 4 * g + (e & 3);
-        sc[e] = key < k_hi ? sa[e >> 2][e & 3] * scale : -INFINITY;
+        sc[e] = key < k_hi ? sa[e >> 2][e & 3] * scale2 : -INFINITY;
         tmax = fmaxf(tmax, sc[e]);
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m_run, tmax);
+      const float m_new = tmax > m_run + kLazyMax ? tmax : m_run;  // the reference moves only on a real jump
       float p[8], tsum = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        p[e] = sc[e] == -INFINITY ? 0.f : expf(sc[e] - m_new);
+        p[e] = sc[e] == -INFINITY ? 0.f : exp2f(sc[e] - m_new);
         tsum += p[e];
       }
       tsum += __shfl_xor(tsum, 16, 64);
       tsum += __shfl_xor(tsum, 32, 64);
-      const float resc = m_run == -INFINITY ? 0.f : expf(m_run - m_new);
+      const float resc = m_run == -INFINITY ? 0.f : exp2f(m_run - m_new);
       m_run = m_new;
       l_run = l_run * resc + tsum;
       pk::u32x4 pw;
@@ -471,7 +647,7 @@ latent_merge_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t out_sh, co
     const float m = in ? ws_ml[(base + static_cast<int64_t>(p) * H) * 2] : -INFINITY;
     const float l = in ? ws_ml[(base + static_cast<int64_t>(p) * H) * 2 + 1] : 0.f;
     const float M = pk::wave_max(m);
-    const float w = m == -INFINITY ? 0.f : expf(m - M);
+    const float w = m == -INFINITY ? 0.f : exp2f(m - M);  // the runs' maxima are in log2 units
     const float L = pk::wave_sum(w * l);
     wgt[p] = L > 0.f ? w / L : 0.f;
   }
@@ -623,6 +799,9 @@ PK_EXPORT int pkm_latent_attention(void* out, long long out_st, long long out_sh
   if (dt == kBF16 && g_latent_mfma && q_st % 8 == 0 && q_sh % 8 == 0 && out_st % 4 == 0 && out_sh % 4 == 0 &&
       reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(cache) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(out) % 8 == 0) {
+    if (R == 512 && cache_t && g_latent_dma)
+      return launch_latent_dma512(out, out_st, out_sh, q, q_st, q_sh, cache, cache_t, block_tables, max_blocks, cu_q,
+                                  context_lens, n_seqs, T, H, block_size, scale, stream);
 #define PKM_LM(RR)                                                                                                 \
   case RR:                                                                                                         \
     return launch_latent_mfma<RR>(out, out_st, out_sh, q, q_st, q_sh, cache, cache_t, block_tables, max_blocks,    \

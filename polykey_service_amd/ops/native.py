@@ -78,6 +78,7 @@ MIXER_SIGNATURES = {
     "pkm_latent_decode": [P, I64, I64, P, I64, I64, P, P, P, I32, P, P, I32, I32, I32, I32, F32, P, P, I32, I32, P],
     "pkm_latent_mfma_rank": [I32],
     "pkm_set_latent_mfma": [I32],
+    "pkm_set_latent_dma": [I32],
     "pkm_gate_merge": [P, P, I64, I64, P, I64, I32, I32, I32, I32, P],
     "pkm_route_sigmoid_topk": [P, P, P, P, I32, I32, I32, I32, P],
     "pkm_expert_gate_up": [P, P, P, P, P, P, P, I32, I32, I32, I32, I32, I32, P],
