@@ -379,3 +379,53 @@ def test_aligned_sizes_on_the_matrix_core_paths(tmp_path):
         err = torch.stack([got[k][p] - want[k][p] for p in range(len(toks))])
         assert float(err.pow(2).mean().sqrt()) < 0.04 * float(want[k].pow(2).mean().sqrt())
         assert float(err.abs().max()) < 0.25 * float(want[k].abs().max())
+
+
+def test_served_over_grpc_with_sampling(small):
+    """The family behind the gRPC tool surface (AsyncLLM loop, tokenizer, sampler): greedy ids equal
+    the plain model's continuation, seeded sampling is reproducible and uses the state slots of
+    several concurrent requests."""
+    import grpc
+
+    from polykey_service_amd import proto
+    from polykey_service_amd.adapters.local_llm import attach_local_llm
+    from polykey_service_amd.config.server_config import ServerConfig
+    from polykey_service_amd.service import ToolRouter
+    from polykey_service_amd.utils import slog
+    from tests.helpers import ServerThread
+
+    cfg, w, path = small
+    eng = LLMEngine(EngineConfig(model_path=path, dtype="float32", max_num_seqs=4, max_num_batched_tokens=64,
+                                 max_model_len=256, num_kv_blocks=32, hip_graphs=False, device="cpu"), ParallelState())
+    router = ToolRouter()
+    attach_local_llm(router, ServerConfig(model="m", model_path=path, backend="local"), slog.Logger(open(os.devnull, "w")),
+                     engine=eng)
+    prompt = rand_tokens(20, cfg["vocab"], 77)
+    seq = list(prompt)
+    for _ in range(6):
+        seq.append(int(O.forward(seq, w, cfg)[-1].argmax()))
+
+    def req(**params):
+        r = proto.ExecuteToolRequest(tool_name="llm.generate")
+        r.parameters.update(params)
+        return r
+
+    try:
+        with ServerThread(router) as s, grpc.insecure_channel(s.addr) as ch:
+            call = ch.unary_unary(proto.EXECUTE_TOOL, request_serializer=proto.ExecuteToolRequest.SerializeToString,
+                                  response_deserializer=proto.ExecuteToolResponse.FromString)
+            r = call(req(prompt_token_ids=prompt, max_tokens=6, ignore_eos=True, return_token_ids=True, **{"return": "struct"}), timeout=120)
+            d = proto.struct_to_dict(r.struct_output)
+            assert [int(t) for t in d["token_ids"]] == seq[len(prompt):], d
+            futs = [call.future(req(prompt_token_ids=rand_tokens(9 + i, cfg["vocab"], i), max_tokens=5, temperature=0.8,
+                                    top_p=0.9, seed=5, ignore_eos=True, return_token_ids=True, **{"return": "struct"}), timeout=120)
+                    for i in range(4)]
+            first = [proto.struct_to_dict(f.result().struct_output)["token_ids"] for f in futs]
+            again = proto.struct_to_dict(call(req(prompt_token_ids=rand_tokens(9, cfg["vocab"], 0), max_tokens=5,
+                                                  temperature=0.8, top_p=0.9, seed=5, ignore_eos=True,
+                                                  return_token_ids=True, **{"return": "struct"}),
+                                              timeout=120).struct_output)["token_ids"]
+            assert again == first[0] and all(len(t) == 5 for t in first)
+    finally:
+        router.llm.shutdown()
+    assert eng.bm.num_free_state_slots == 4
