@@ -370,8 +370,13 @@ latent_attention_mfma_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t o
 // tile t's products run, one barrier per tile.  A wave instruction moves 1 KiB: exactly one
 // key-major row (padded to 1040 B in LDS through the instruction's LDS base), or 16 rows of the
 // latent-major copy, whose 16-byte parts are XOR-swizzled by the row on the GLOBAL side of the
-// copy (lane l fetches part (l & 3) ^ ((l >> 3) & 3) of row l >> 2) so that the unpadded 64-byte
-// rows read conflict-free.  Needs the latent-major cache copy (pages of whole 32-key tiles).
+// copy (lane l fetches part (l & 3) ^ part_swizzle(l >> 2) of row l >> 2) so that the unpadded
+// 64-byte rows read conflict-free.  Needs the latent-major cache copy (pages of whole 32-key tiles).
+// part_swizzle(r) = (r2, r3 ^ r1) as (low, high) bit: a fragment read takes 16 rows at one part,
+// and the 16 rows' 16-byte parts then fall on 16 different 16-byte bank groups whether the LDS
+// serves 8 lanes over 32 banks or 16 lanes over 64 banks per pass.
+__device__ __forceinline__ int part_swizzle(int r) { return ((r >> 2) & 1) | ((((r >> 3) ^ (r >> 1)) & 1) << 1); }
+
 __global__ void __launch_bounds__(kPromptThreads)
 latent_attention_dma512_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t out_sh, const bf16_t* __restrict__ q,
                                int64_t q_st, int64_t q_sh, const bf16_t* __restrict__ cache,
@@ -417,7 +422,7 @@ latent_attention_dma512_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t
 
   // lane offsets of the two copies: key-major rows are taken as they lie, latent-major parts swizzled
   const unsigned kvo = static_cast<unsigned>(lane) * 16u;
-  const unsigned tvo = static_cast<unsigned>(((lane >> 2) * 4 + ((lane & 3) ^ ((lane >> 3) & 3))) * 16);
+  const unsigned tvo = static_cast<unsigned>(((lane >> 2) * 4 + ((lane & 3) ^ part_swizzle(lane >> 2))) * 16);
   auto issue = [&](int k0, int buf) {  // this wave's 4 + 4 KiB of the tile at k0
     const int blk = __builtin_amdgcn_readfirstlane(bt[k0 / block_size]);
     const int kin = k0 % block_size;
@@ -483,7 +488,7 @@ latent_attention_dma512_kernel(bf16_t* __restrict__ out, int64_t out_st, int64_t
         for (int rt = 0; rt < NRT; ++rt) o[rt] *= resc;
       }
       // row rt*16 + n of the latent-major tile, part g, at its swizzled place
-      const bf16_t* vr = ct + (n * 4 + (g ^ ((n >> 1) & 3))) * 8;
+      const bf16_t* vr = ct + (n * 4 + (g ^ part_swizzle(n))) * 8;
 #pragma unroll
       for (int rt = 0; rt < NRT; ++rt)
         o[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(vr + rt * 16 * 32), pb, o[rt], 0, 0, 0);

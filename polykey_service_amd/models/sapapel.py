@@ -26,8 +26,6 @@ implemented for this family (the layers are a few megabytes to a few hundred: on
 """
 from __future__ import annotations
 
-import json
-import os
 from typing import List, Optional
 
 import torch
@@ -338,7 +336,3 @@ class SapapelForCausalLM(nn.Module):
                                           act_dtype=self.dtype)
         return gemm.linear(act, self.head).float()
 
-
-def config_from_dir(path: str) -> SapapelConfig:
-    with open(os.path.join(path, "config.json")) as f:
-        return SapapelConfig.from_json(json.load(f), os.path.basename(os.path.abspath(path)))
