@@ -139,6 +139,8 @@ class ModelRunner:
             self.part_o = self.part_ml = None
             if hasattr(model, "reserve_steps"):
                 model.reserve_steps(self.max_step_tokens)
+            if hasattr(model, "reserve_positions"):  # position tables (rotations) up to the longest sequence
+                model.reserve_positions(cfg.max_model_len)
         else:
             a0 = model.layers[0].attn
             self.part_o, self.part_ml = attn_ops.decode_workspace(cfg.max_num_seqs, a0.nq, self.max_blocks, self.bs,

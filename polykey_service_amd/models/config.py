@@ -107,8 +107,8 @@ class SigmoidMoESpec:
 @dataclasses.dataclass(frozen=True)
 class LayerSpec:
     type: str
-    mixer: LatentAttentionSpec
-    mlp: Optional[SigmoidMoESpec]
+    mixer: object    # the mixer's spec (LatentAttentionSpec, SinkAttentionSpec, LightningSpec)
+    mlp: object      # the feed-forward's spec, None: no feed-forward
 
 
 @dataclasses.dataclass(frozen=True)
@@ -175,8 +175,176 @@ class SapapelConfig:
         return cls(name=name, vocab_size=vocab, hidden_size=width, layers=(l,) * n_layers, alpha=alpha, rms_eps=eps)
 
 
+@dataclasses.dataclass(frozen=True)
+class RotarySpec:
+    """Rotation of interleaved coordinate pairs (2i, 2i+1) of the first ``dims`` coordinates by
+    position * base^(-2i/dims); ``scaling`` = (factor, original, fast, slow) stretches the slow
+    pairs (YaRN) and scales cos / sin by 0.1 ln(factor) + 1."""
+    dims: int
+    base: float
+    scaling: Optional[tuple] = None
+
+
+@dataclasses.dataclass(frozen=True)
+class SinkAttentionSpec:
+    """Grouped-query softmax attention with unit-RMS rotated queries / keys, position-rotated values,
+    a tanh cap on the scores (0: none) and ``sink`` extra exp(0) terms in the softmax denominator."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    softcap: float = 0.0
+    rot: Optional[RotarySpec] = None
+    sink: float = 1.0
+
+
+@dataclasses.dataclass(frozen=True)
+class LightningSpec:
+    """Linear attention with one constant decay per head and a [dim, vdim] fp32 state per head."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+
+
+@dataclasses.dataclass(frozen=True)
+class DenseFFSpec:
+    ff: int
+
+
+@dataclasses.dataclass(frozen=True)
+class ClampedMoESpec:
+    """Experts with clamped gate / up products, chosen by the largest router logits and weighted by
+    the softmax over the chosen logits; optionally one shared expert behind a sigmoid gate."""
+    experts: int
+    top: int
+    ff: int
+    limit: float
+    shared_ff: int = 0
+    shared_limit: float = 0.0
+
+
+@dataclasses.dataclass(frozen=True)
+class KivezenConfig:
+    """Kivezen: pre-norm layers on ``streams`` fp32 residual streams (hyper-connections; 0: the one
+    plain residual), each layer a sink-softmax attention or a lightning (decayed linear) attention
+    mixer and a dense GELU or clamped-GLU MoE feed-forward; layers ``loop[0]..loop[1]-1`` run
+    ``loop[2]`` times in a row with the same weights and a cache / state per pass.  Read from a
+    checkpoint folder's config.json ("architecture": "Kivezen")."""
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple
+    rms_eps: float
+    streams: int = 0
+    loop: tuple = (0, 0, 1)
+    logit_softcap: float = 0.0
+    max_position: int = 1 << 20     # the rotation tables are built for the engine's max_model_len
+    bos_token_id: int = 0
+    eos_token_id: int = -1
+    init_std: float = 0.05
+    family: str = "kivezen"
+    is_moe: bool = False            # not the Mixtral expert-parallel family (engine lockstep paths)
+    experts_per_token: int = 0
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def runs(self) -> tuple:
+        """Layer index of every layer run, in execution order (a looped layer appears once per pass)."""
+        a, b, times = self.loop
+        n = len(self.layers)
+        return tuple(range(a)) + tuple(range(a, b)) * times + tuple(range(b, n))
+
+    @property
+    def needs_state(self) -> bool:
+        return any(l.type == "lightning" for l in self.layers)
+
+    def num_params(self) -> int:
+        W, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size
+        for l in self.layers:
+            m = l.mixer
+            if l.type == "attention":
+                n += W * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim) + m.heads * m.vdim)
+            else:
+                n += W * m.heads * (2 * m.dim + 3 * m.vdim)
+            f = l.mlp
+            if isinstance(f, DenseFFSpec):
+                n += 2 * W * f.ff
+            elif f is not None:
+                n += f.experts * (3 * f.ff * W + W) + 3 * f.shared_ff * W
+        return n
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        return sum(self.layers[i].mixer.kv_heads * (self.layers[i].mixer.dim + self.layers[i].mixer.vdim)
+                   for i in self.runs if self.layers[i].type == "attention") * dtype_bytes
+
+    @classmethod
+    def from_json(cls, c: dict, name: str = "kivezen") -> "KivezenConfig":
+        layers = []
+        for l in c["layers"]:
+            m = l["mixer"]
+            if l["type"] == "attention":
+                rot = None
+                if m.get("rot"):
+                    sc = m["rot"].get("scaling")
+                    rot = RotarySpec(int(m["rot"]["dims"]), float(m["rot"]["base"]),
+                                     (float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"]))
+                                     if sc else None)
+                mixer = SinkAttentionSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]),
+                                          int(m.get("vdim", m["dim"])), float(m["scale"]), float(m.get("softcap") or 0.0),
+                                          rot)
+            elif l["type"] == "lightning":
+                mixer = LightningSpec(int(m["heads"]), int(m["dim"]), int(m.get("vdim", m["dim"])),
+                                      tuple(float(d) for d in m["decay"]))
+                if len(mixer.decay) != mixer.heads:
+                    raise ValueError("Kivezen: a lightning mixer needs one decay per head")
+            else:
+                raise ValueError(f"Kivezen: unknown mixer type {l['type']!r}")
+            f = l.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind") == "dense":
+                    mlp = DenseFFSpec(int(f["ff"]))
+                elif f.get("kind") == "moe":
+                    sh = f.get("shared") or {}
+                    mlp = ClampedMoESpec(int(f["router"]["experts"]), int(f["router"]["top"]), int(f["expert"]["ff"]),
+                                         float(f["expert"]["limit"]), int(sh.get("ff", 0)), float(sh.get("limit", 0.0)))
+                else:
+                    raise ValueError(f"Kivezen: unknown feed-forward kind {f.get('kind')!r}")
+            layers.append(LayerSpec(l["type"], mixer, mlp))
+        lp = c.get("loop") or {}
+        loop = (int(lp.get("start", 0)), int(lp.get("stop", 0)), int(lp.get("times", 1)))
+        if not (0 <= loop[0] <= loop[1] <= len(layers)) or loop[2] < 1:
+            raise ValueError(f"Kivezen: loop {loop} does not fit {len(layers)} layers")
+        return cls(name=name, vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), layers=tuple(layers),
+                   rms_eps=float(c["norm"]["eps"]), streams=int(c.get("streams") or 0), loop=loop,
+                   logit_softcap=float(c.get("logit_softcap") or 0.0))
+
+    @classmethod
+    def uniform(cls, name: str, vocab: int, width: int, pattern: str, heads: int, kv_heads: int, dim: int, ff: int,
+                experts: int, top: int, expert_ff: int, streams: int = 2, loop: tuple = (0, 0, 1)) -> "KivezenConfig":
+        """``pattern``: one letter per layer, A attention / L lightning, upper case with the MoE
+        feed-forward (and a shared expert of ``expert_ff``), lower case with the dense one."""
+        rot = RotarySpec(dim, 10000.0, (8.0, 4096.0, 32.0, 1.0))
+        layers = []
+        for ch in pattern:
+            if ch in "Aa":
+                mixer = SinkAttentionSpec(heads, kv_heads, dim, dim, dim ** -0.5, 30.0, rot)
+            else:
+                mixer = LightningSpec(heads, dim, dim, tuple(1.0 - 2.0 ** (-1 - 6 * h / max(heads - 1, 1))
+                                                             for h in range(heads)))
+            mlp = ClampedMoESpec(experts, top, expert_ff, 7.0, expert_ff, 7.0) if ch.isupper() else DenseFFSpec(ff)
+            layers.append(LayerSpec("attention" if ch in "Aa" else "lightning", mixer, mlp))
+        return cls(name=name, vocab_size=vocab, hidden_size=width, layers=tuple(layers), rms_eps=1e-5,
+                   streams=streams, loop=loop, logit_softcap=50.0)
+
+
 # config.json "architecture" -> reader (checkpoints that are not HF Llama / Mixtral folders)
-ARCHITECTURES = {"Sapapel": SapapelConfig.from_json}
+ARCHITECTURES = {"Sapapel": SapapelConfig.from_json, "Kivezen": KivezenConfig.from_json}
 
 PRESETS["tiny-sapapel"] = SapapelConfig.uniform("tiny-sapapel", 512, 128, 3, 4, 16, 32, 48, 64, 6, 2)
 # speed measurements (random weights): layer shapes of small production MoE models, and the
@@ -187,6 +355,13 @@ PRESETS["mixtral-2k"] = ModelConfig("mixtral-2k", 32000, 2048, 1536, 8, 16, 4, r
                                     experts_per_token=2, bos_token_id=1, eos_token_id=2, router_init_std=0.5)
 PRESETS["mixtral-4k"] = ModelConfig("mixtral-4k", 32000, 4096, 2048, 4, 32, 8, rope_theta=1e6, num_experts=8,
                                     experts_per_token=2, bos_token_id=1, eos_token_id=2, router_init_std=0.5)
+
+
+PRESETS["tiny-kivezen"] = KivezenConfig.uniform("tiny-kivezen", 512, 128, "LAa", 4, 2, 32, 256, 6, 2, 64, loop=(1, 3, 2))
+# speed measurements beside mixtral-2k / mixtral-4k: the same width, depth, heads, KV heads, experts
+# and expert size; every fourth mixer is a lightning layer, every layer has the MoE with a shared expert
+PRESETS["kivezen-2k"] = KivezenConfig.uniform("kivezen-2k", 32000, 2048, "LAAALAAA", 16, 4, 128, 4096, 16, 2, 1536)
+PRESETS["kivezen-4k"] = KivezenConfig.uniform("kivezen-4k", 32000, 4096, "LAAA", 32, 8, 128, 8192, 8, 2, 2048)
 
 
 def get_config(name_or_path: str):

@@ -316,3 +316,120 @@ def input_scaled_moe(x: torch.Tensor, x_act: torch.Tensor, ids: torch.Tensor, wt
         return y, inv
     native.call("pkm_combine_rows", out.data_ptr(), y.data_ptr(), inv.data_ptr(), T, k, W, 1, st)
     return out
+
+
+# ------------------------------------------------------------------ logit-routed experts with clamped products
+ROUTER_KERNEL_MAX_T = 256
+
+
+def router_logits(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x [T, W] fp32 times w [N, W] fp32 -> [T, N] fp32 in true fp32.  Decode-sized steps on the GPU take
+    one wave per (token, row); larger ones an fp32 library GEMM."""
+    if not x.is_cuda or x.shape[0] > ROUTER_KERNEL_MAX_T:
+        return torch.mm(x, w.t())
+    assert x.dtype == torch.float32 and w.dtype == torch.float32 and x.is_contiguous() and w.is_contiguous()
+    out = torch.empty((x.shape[0], w.shape[0]), dtype=torch.float32, device=x.device)
+    native.call("pkm_router_logits", out.data_ptr(), x.data_ptr(), w.data_ptr(), x.shape[0], w.shape[0], x.shape[1],
+                native.stream_ptr())
+    return out
+
+
+def route_topk_softmax(logits: torch.Tensor, E: int, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp32 router logits [T, >= E] (the first E columns of each row; the row may hold more) -> the k
+    experts with the largest logits (ties: the lower expert id) and the softmax over those k logits."""
+    T = logits.shape[0]
+    if not logits.is_cuda:
+        z, ids = torch.sort(logits[:, :E].float(), dim=-1, descending=True, stable=True)
+        return ids[:, :k].to(torch.int32).contiguous(), torch.softmax(z[:, :k], -1).contiguous()
+    assert logits.dtype == torch.float32 and logits.stride(1) == 1
+    ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+    native.call("pkm_route_topk_softmax", ids.data_ptr(), w.data_ptr(), logits.data_ptr(), logits.stride(0), T, E, k,
+                native.stream_ptr())
+    return ids, w
+
+
+def _clamped(g: torch.Tensor, u: torch.Tensor, limit: float) -> torch.Tensor:
+    g = g.clamp(max=limit)
+    u = u.clamp(-limit, limit)
+    return g * torch.sigmoid(1.702 * g) * (u + 1)
+
+
+def clamped_glu(gu, limit: float, interleaved: bool = False, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """gu [n, 2F]: gate products then up products (``interleaved``: alternating in blocks of 16, the
+    layout of the grouped MFMA GEMMs) -> min(g, limit) * sigmoid(1.702 min(g, limit)) * (clamp(u) + 1).
+    ``gu`` may be the decode GEMM's unreduced split-K slabs (``gemm.Partial``): their sum is taken on
+    the way in and the result is written in ``dtype``."""
+    if isinstance(gu, gemm.Partial):
+        out = torch.empty((gu.M, gu.N // 2), dtype=dtype, device=gu.buf.device)
+        native.call("pkm_clamped_glu_slabs", out.data_ptr(), gu.buf.data_ptr(), gu.S, gu.M, gu.N // 2, float(limit),
+                    int(interleaved), native.dt_code(dtype), native.stream_ptr())
+        return out
+    n, F2 = gu.shape
+    F_ = F2 // 2
+    if not gu.is_cuda:
+        f = gu.float()
+        if interleaved:
+            v = f.view(n, F_ // 16, 2, 16)
+            g, u = v[:, :, 0].reshape(n, F_), v[:, :, 1].reshape(n, F_)
+        else:
+            g, u = f[:, :F_], f[:, F_:]
+        return _clamped(g, u, limit).to(gu.dtype)
+    out = torch.empty((n, F_), dtype=gu.dtype, device=gu.device)
+    assert gu.is_contiguous() and (not interleaved or F_ % 16 == 0)
+    native.call("pkm_clamped_glu", out.data_ptr(), gu.data_ptr(), n, F_, float(limit), int(interleaved),
+                native.dt_code(gu.dtype), native.stream_ptr())
+    return out
+
+
+def gelu_tanh(x: torch.Tensor) -> torch.Tensor:
+    """0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))), fp32 maths, in place."""
+    if not x.is_cuda:
+        return x.copy_(F.gelu(x.float(), approximate="tanh"))
+    assert x.is_contiguous()
+    native.call("pkm_gelu_tanh", x.data_ptr(), x.numel(), native.dt_code(x.dtype), native.stream_ptr())
+    return x
+
+
+def clamped_experts(x_act: torch.Tensor, ids: torch.Tensor, gate, up, down, limit: float, w13=None, w2=None,
+                    w13_p=None, w2_p=None):
+    """Rows of every (token, chosen expert) pair through the expert's clamped GLU: (y [T * top, W] in
+    expert order, inv [T * top]) for the kernel that sums them with the routing weights.  With
+    ``w13`` / ``w2`` (shapes of :func:`mfma_experts_ok`) the framework's grouped MFMA GEMMs, else
+    gate / up [E, F, W], down [E, W, F] through the tiled FMA grouped kernels (any sizes, fp32 too)."""
+    T, W = x_act.shape
+    k = ids.shape[1]
+    n = T * k
+    if w13 is not None:
+        E = w13.shape[0]
+        offsets, sorted_, inv = align(ids, E, 0, E)
+        if T <= 64 and E <= 64 and gemm.SKINNY_ENABLED:  # decode: the GEMM gathers the tokens' rows itself
+            gu = gemm.grouped_linear(x_act, w13, offsets, T, False, packed=w13_p, a_rows=sorted_, a_row_div=k, n_rows=n)
+            return gemm.grouped_linear(clamped_glu(gu, limit, interleaved=True), w2, offsets, T, False, packed=w2_p), inv
+        xs = permute(x_act, sorted_, offsets, k)
+        gu = grouped_gemm(xs, w13, offsets, T, silu=False, packed=w13_p)
+        y = grouped_gemm(clamped_glu(gu, limit, interleaved=True), w2, offsets, T, silu=False, packed=w2_p)
+        return y, inv
+    E, F_, _ = gate.shape
+    offsets, sorted_, inv = align(ids, E, 0, E)
+    if not x_act.is_cuda:
+        m = int(offsets[-1])
+        tok = sorted_[:m].long() // k
+        y = torch.zeros((m, W), dtype=torch.float32)
+        offs = offsets.tolist()
+        for e in range(E):
+            lo, hi = offs[e], offs[e + 1]
+            if hi > lo:
+                xe = x_act[tok[lo:hi]]
+                h = _clamped(F.linear(xe, gate[e]).float(), F.linear(xe, up[e]).float(), limit).to(x_act.dtype)
+                y[lo:hi] = F.linear(h, down[e]).float()
+        return y, inv
+    assert x_act.is_contiguous() and gate.is_contiguous() and up.is_contiguous() and down.is_contiguous()
+    dt = native.dt_code(x_act.dtype)
+    h = torch.empty((n, F_), dtype=x_act.dtype, device=x_act.device)
+    y = torch.empty((n, W), dtype=torch.float32, device=x_act.device)
+    st = native.stream_ptr()
+    native.call("pkm_expert_gate_up_clamped", h.data_ptr(), x_act.data_ptr(), gate.data_ptr(), up.data_ptr(),
+                offsets.data_ptr(), sorted_.data_ptr(), float(limit), n, k, E, F_, W, dt, st)
+    native.call("pkm_expert_down", y.data_ptr(), h.data_ptr(), down.data_ptr(), offsets.data_ptr(), n, E, W, F_, dt, st)
+    return y, inv

@@ -86,6 +86,22 @@ MIXER_SIGNATURES = {
     "pkm_combine_rows": [P, P, P, I32, I32, I32, I32, P],
     "pkm_permute_scaled": [P, P, P, P, I32, I32, I32, I32, P],
     "pkm_expert_align_wide": [P, P, P, P, I32, I32, P],
+    "pkm_expert_gate_up_clamped": [P, P, P, P, P, P, F32, I32, I32, I32, I32, I32, I32, P],
+    "pkm_spread_rows": [P, P, P, I32, I32, I32, I32, I32, P],
+    "pkm_hyper_step": [P, I32, I32, I32, P, I32, I32, P, I32, P, P, I32, P, I64, P, P, P, P, F32, P, I32, P, P, P],
+    "pkm_tanh_cap": [P, I64, F32, P],
+    "pkm_route_topk_softmax": [P, P, P, I64, I32, I32, I32, P],
+    "pkm_router_logits": [P, P, P, I32, I32, I32, P],
+    "pkm_clamped_glu": [P, P, I32, I32, F32, I32, I32, P],
+    "pkm_clamped_glu_slabs": [P, P, I32, I32, I32, F32, I32, I32, P],
+    "pkm_gelu_tanh": [P, I64, I32, P],
+    "pkm_gated_rms_norm": [P, P, P, P, I64, I32, I32, F32, I32, I32, P],
+    "pkm_lightning_attention": [P, P, I64, P, P, P, P, P, I32, I32, I32, I32, I32, I32, I32, P],
+    "pkm_rope_norm_cache": [P, P, I64, I32, P, P, P, I32, P, I32, P, P, I32, I32, I32, I32, I32, I32, F32, I32, P],
+    "pkm_sink_decode_part": [I32, I32, I32, I32, I32],
+    "pkm_set_sink_mfma": [I32],
+    "pkm_sink_attention": [P, P, P, P, P, I64, P, P, P, P, P, I32, I32, I32, I32, I32, I32, I32, I32, F32, F32, I32,
+                           P, P, I32, I32, I32, P],
 }
 _mixers: Optional[ctypes.CDLL] = None
 
