@@ -94,13 +94,14 @@ __device__ __forceinline__ bool find_tile(const int* offsets, int E, int tile, i
   return false;
 }
 
-// C[r, n] = sum_k A[arow(r), k] * B[e][n, k]   (B: [E, N, K]); DUAL: a second B and the scaled
-// SiLU-product epilogue.  256 threads: thread (ty, tx) owns rows ty, ty + 16 and columns tx, tx + 16.
+// C[r, n] = sum_k A[arow(r), k] * B[e][n, k]   (B: [E, N, K]); DUAL: a second B and a gated
+// epilogue: with slot_scale the scaled SiLU product, without it the clamped product
+// min(g, limit) * sigmoid(1.702 min(g, limit)) * (clamp(u, -limit, limit) + 1).  256 threads: thread (ty, tx) owns rows ty, ty + 16 and columns tx, tx + 16.
 template <typename T, typename TA, typename TC, bool DUAL>
 __global__ void __launch_bounds__(256)
 grouped_rows_kernel(TC* __restrict__ C, const TA* __restrict__ A, const T* __restrict__ B0, const T* __restrict__ B1,
                     const int* __restrict__ offsets, const int* __restrict__ sorted_slots,
-                    const float* __restrict__ slot_scale, int top, int E, int N, int K) {
+                    const float* __restrict__ slot_scale, int top, int E, int N, int K, float limit) {
   __shared__ float as[kBM][kBK + 1];
   __shared__ float b0s[kBN][kBK + 1];
   __shared__ float b1s[DUAL ? kBN : 1][kBK + 1];
@@ -150,15 +151,18 @@ grouped_rows_kernel(TC* __restrict__ C, const TA* __restrict__ A, const T* __res
   for (int i = 0; i < 2; ++i) {
     const int r = r0 + ty + 16 * i;
     if (r >= r1) continue;
-    const float s = DUAL ? slot_scale[sorted_slots[r]] : 1.f;
+    const float s = (DUAL && slot_scale) ? slot_scale[sorted_slots[r]] : 1.f;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int n = n0 + tx + 16 * j;
       if (n >= N) continue;
       float v = acc0[i][j];
-      if (DUAL) {
+      if (DUAL && slot_scale) {
         const float g = s * v, u = s * acc1[i][j];
         v = g * sigmoidf(g) * u;
+      } else if (DUAL) {
+        const float g = fminf(v, limit), u = fminf(fmaxf(acc1[i][j], -limit), limit);
+        v = g * sigmoidf(1.702f * g) * (u + 1.f);
       }
       st<TC>(C + static_cast<int64_t>(r) * N + n, v);
     }
@@ -248,7 +252,21 @@ PK_EXPORT int pkm_expert_gate_up(void* h, const void* x, const void* gate, const
   PKM_DISPATCH(dt, T, grouped_rows_kernel<T, T, T, true><<<grid, 256, 0, stream>>>(
                           static_cast<T*>(h), static_cast<const T*>(x), static_cast<const T*>(gate),
                           static_cast<const T*>(up), static_cast<const int*>(offsets),
-                          static_cast<const int*>(sorted_slots), static_cast<const float*>(slot_scale), top, E, F, W));
+                          static_cast<const int*>(sorted_slots), static_cast<const float*>(slot_scale), top, E, F, W,
+                          0.f));
+  return PK_CHECK_LAUNCH();
+}
+
+// the same with the clamped epilogue (no scores): h = min(g, limit) sigmoid(1.702 min(g, limit)) (clamp(u) + 1)
+PK_EXPORT int pkm_expert_gate_up_clamped(void* h, const void* x, const void* gate, const void* up, const void* offsets,
+                                         const void* sorted_slots, float limit, int n_rows, int top, int E, int F,
+                                         int W, int dt, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  const dim3 grid((n_rows + kBM - 1) / kBM + E, (F + kBN - 1) / kBN);
+  PKM_DISPATCH(dt, T, grouped_rows_kernel<T, T, T, true><<<grid, 256, 0, stream>>>(
+                          static_cast<T*>(h), static_cast<const T*>(x), static_cast<const T*>(gate),
+                          static_cast<const T*>(up), static_cast<const int*>(offsets),
+                          static_cast<const int*>(sorted_slots), nullptr, top, E, F, W, limit));
   return PK_CHECK_LAUNCH();
 }
 
@@ -259,7 +277,7 @@ PK_EXPORT int pkm_expert_down(void* y, const void* h, const void* down, const vo
   const dim3 grid((n_rows + kBM - 1) / kBM + E, (W + kBN - 1) / kBN);
   PKM_DISPATCH(dt, T, grouped_rows_kernel<T, T, float, false><<<grid, 256, 0, stream>>>(
                           static_cast<float*>(y), static_cast<const T*>(h), static_cast<const T*>(down), nullptr,
-                          static_cast<const int*>(offsets), nullptr, nullptr, 1, E, W, F));
+                          static_cast<const int*>(offsets), nullptr, nullptr, 1, E, W, F, 0.f));
   return PK_CHECK_LAUNCH();
 }
 
