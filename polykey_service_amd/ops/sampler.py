@@ -22,6 +22,7 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     if not logits.is_cuda:
         return reference.sample(logits, temperature, top_k, top_p, min_p, seeds, offsets).to(torch.int32)
     assert logits.stride(-1) == 1
+    logits, V = _eight_wide(logits)
     if out is None:
         out = torch.empty(B, dtype=torch.int32, device=logits.device)
     dtype = 0 if logits.dtype == torch.bfloat16 else 1
@@ -32,10 +33,23 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     return out
 
 
+def _eight_wide(logits: torch.Tensor):
+    """The kernel reads rows in 16-byte pieces: a vocabulary (or row stride) that is not a multiple
+    of 8 is copied into rows padded with -inf, which no rule ever picks."""
+    B, V = logits.shape
+    if V % 8 == 0 and logits.stride(0) % 8 == 0:
+        return logits, V
+    Vp = (V + 7) // 8 * 8
+    padded = torch.full((B, Vp), float("-inf"), dtype=logits.dtype, device=logits.device)
+    padded[:, :V] = logits
+    return padded, Vp
+
+
 def greedy(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     if not logits.is_cuda:
         return torch.argmax(logits.float(), dim=-1).to(torch.int32)
-    B, V = logits.shape
+    B = logits.shape[0]
+    logits, V = _eight_wide(logits)
     if out is None:
         out = torch.empty(B, dtype=torch.int32, device=logits.device)
     dtype = 0 if logits.dtype == torch.bfloat16 else 1
