@@ -101,8 +101,10 @@ def parse_args(argv=None):
                          "JSON line is always printed in time")
     ap.add_argument("--compare-families", default="",
                     help="instead of the headline workload: engine-level prefill and decode throughput of the "
-                         "Sapapel family beside the Mixtral family at equal layer sizes, e.g. '2k,4k' "
-                         "(presets sapapel-<size> / mixtral-<size>; random weights, one GPU, no RPC)")
+                         "--compare-family family beside the Mixtral family at equal layer sizes, e.g. '2k,4k' "
+                         "(presets <family>-<size> / mixtral-<size>; random weights, one GPU, no RPC)")
+    ap.add_argument("--compare-family", default="sapapel",
+                    help="--compare-families: the family measured beside the Mixtral family (sapapel, kivezen)")
     ap.add_argument("--compare-batch", type=int, default=32, help="--compare-families: sequences")
     ap.add_argument("--compare-prompt", type=int, default=1024, help="--compare-families: prompt tokens per sequence")
     ap.add_argument("--compare-decode", type=int, default=128, help="--compare-families: decoded tokens per sequence")
@@ -486,7 +488,7 @@ def compare_families(args) -> int:
     rng = __import__("random").Random(args.seed)
     for item in [x for x in args.compare_families.split(",") if x]:
         size, _, only = item.partition(":")  # "2k" both families, "2k:sapapel" one (profiling)
-        for fam in ((only,) if only else ("sapapel", "mixtral")):
+        for fam in ((only,) if only else (args.compare_family, "mixtral")):
             name = f"{fam}-{size}"
             eng = LLMEngine(EngineConfig(model=name, seed=args.seed, max_num_seqs=B,
                                          max_num_batched_tokens=args.max_batched_tokens, max_model_len=max_len,
@@ -494,7 +496,8 @@ def compare_families(args) -> int:
                                          num_kv_blocks=B * (max_len // 32) + 16), ParallelState(device=dev))
             V = eng.mcfg.vocab_size
             prompts = [[rng.randrange(3, V) for _ in range(S)] for _ in range(B)]
-            eng.generate([p[:96] for p in prompts[:2]], SamplingParams(max_tokens=4, ignore_eos=True))  # warm-up
+            # warm-up: a prompt-sized step (library GEMM paths, lazily loaded kernels) and a few decode steps
+            eng.generate([p[:min(S, 320)] for p in prompts[:2]], SamplingParams(max_tokens=4, ignore_eos=True))
             torch.cuda.synchronize(dev)
             t0 = time.perf_counter()
             eng.generate(prompts, SamplingParams(max_tokens=1, ignore_eos=True))
